@@ -1,0 +1,106 @@
+"""Configuration container of the gfx950 FlashAttention-2 kernels.
+
+Mirrors ``KernelsConfigV2`` and ``init_to_zero_v2`` of the reference
+(src/flash_attention_triton/_configurators_v2.py:9-93) so that code written against
+``flash_attention_v2_custom`` keeps working, without importing Triton.  The fields keep their
+names; what they select here is a row of the gfx950 tile/wave table compiled into
+``libfa2_gfx950.so`` rather than Triton meta-parameters.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Callable
+from dataclasses import dataclass, field
+from typing import Any
+
+import torch
+
+
+@dataclass(frozen=True)
+class BackwardConfig:
+    """Stand-in for ``triton.Config`` in ``backward_autotune_configs``.
+
+    Any object with the same attributes (``kwargs``, ``num_warps``, ``num_stages``,
+    ``pre_hook``) is accepted, a real ``triton.Config`` included.  Only
+    ``kwargs["SEQUENCE_PARALLEL"]`` changes behaviour: it selects the non-deterministic
+    backward (reference: flash_attention_2.py:204-207, _triton_kernels_v2.py:466-525).
+    """
+
+    kwargs: dict[str, Any]
+    num_warps: int = 4
+    num_stages: int = 2
+    pre_hook: Callable[..., Any] | None = None
+
+    def __hash__(self) -> int:  # dict field: hash by content
+        return hash((tuple(sorted(self.kwargs.items())), self.num_warps, self.num_stages))
+
+
+@dataclass(frozen=True)
+class KernelsConfigV2:
+    """Configuration container for the FlashAttention-2 kernels (reference: _configurators_v2.py:9-38).
+
+    Attributes:
+        block_rows_size: Query rows per workgroup in the forward kernel (the compiled kernels
+            use 128; other values are accepted and ignored).
+        block_cols_size: Key rows per inner step of the forward kernel (compiled: 64).
+        min_block_headdim: Smallest padded head dimension (power of two, at least 16).
+        max_headdim: Largest supported head dimension.  Also the multiple to which the
+            log-sum-exp row length is padded (reference: flash_attention_2.py:98).
+        seqlen_cache_divisor: Kept for signature compatibility; the reference uses it to bound
+            Triton recompilation, which does not exist here.
+        min_warps: Wavefronts (64 lanes) per workgroup.
+        max_warps: Kept for signature compatibility (dead in the reference as well).
+        num_stages: LDS stages of the streamed tiles (compiled: 2).
+        backward_autotune_configs: Backward configurations; the backward is deterministic
+            unless one of them sets ``SEQUENCE_PARALLEL`` to True.
+    """
+
+    block_rows_size: int
+    block_cols_size: int
+    min_block_headdim: int
+    max_headdim: int
+    seqlen_cache_divisor: int
+    min_warps: int
+    max_warps: int
+    num_stages: int
+    backward_autotune_configs: list = field(default_factory=list)
+
+    def _create_kernel_key(self) -> tuple[tuple[int, int], tuple]:
+        """Immutable key: (compute capability of the current device, all field values).
+
+        Same role as the reference's backward-kernel cache key (_configurators_v2.py:40-55).
+        """
+        cc = torch.cuda.get_device_capability()
+
+        def _serialize(name: str) -> object:
+            attr = getattr(self, name)
+            return self._serialize_bwd(attr) if name == "backward_autotune_configs" else attr
+
+        return cc, tuple(_serialize(name) for name in self.__annotations__)
+
+    def _serialize_bwd(self, bwd_configs: list) -> tuple:
+        """Hashable form of the backward configurations (reference: _configurators_v2.py:57-73)."""
+        return tuple(
+            (tuple(c.kwargs.values()), c.num_warps, c.num_stages, self._hook_name(c.pre_hook))
+            for c in bwd_configs
+        )
+
+    @staticmethod
+    def _hook_name(pre_hook: object) -> str | None:
+        return getattr(pre_hook, "__qualname__", None)
+
+    @property
+    def deterministic(self) -> bool:
+        """True unless a backward configuration asks for sequence-parallel dQ accumulation."""
+        return not any(bool(getattr(c, "kwargs", {}).get("SEQUENCE_PARALLEL", False))
+                       for c in self.backward_autotune_configs)
+
+
+def init_to_zero_v2(name: str) -> Callable[[dict[str, torch.Tensor]], torch.Tensor]:
+    """Pre-hook that zeroes the tensor called ``name`` in a kernel-argument dictionary.
+
+    Same contract as the reference (_configurators_v2.py:81-93).  The gfx950 library clears its
+    own dQ workspace when a mode needs one, so the hook is never called by this package; it is
+    kept so that configurations written for the reference still construct.
+    """
+    return lambda nargs: nargs[name].zero_()

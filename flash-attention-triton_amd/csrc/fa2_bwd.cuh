@@ -1,0 +1,467 @@
+// Causal FlashAttention-2 backward for gfx950.
+//
+// The reference backward (src/flash_attention_triton/_triton_kernels_v2.py:192-352) walks, for
+// one key/value tile j, all query tiles i at or below the diagonal and does
+//   S = Q_i K_j^T,  P = exp(scale*S - lse_i),  dP = dO_i V_j^T,  dS = P*(dP - delta_i)*scale,
+//   dK_j += dS^T Q_i,  dV_j += P^T dO_i,  dQ_i += dS K_j
+// with dQ either atomically added (sequence-parallel) or read-modify-written by a single
+// sequential program per head (deterministic).  Here the work is split so that every output is
+// owned by exactly one wave and written once:
+//
+//  * bwd_dkdv_kernel: one workgroup per key/value tile of 128 rows, each of its 4 waves owning 32
+//    key columns (K and V fragments stay in registers); Q and dO tiles stream through LDS.
+//    S and dP come out of the MFMA with one key column per lane, which is the B-operand layout
+//    dV^T = dO^T P and dK^T = Q^T dS need; dO^T and Q^T fragments are fetched from the row-major
+//    tiles with the transposing LDS read.
+//  * bwd_dq_kernel: one workgroup per query tile of 128 rows, each wave owning 32 query columns
+//    (Q and dO fragments in registers); K and V tiles stream through LDS in ascending order.  It
+//    recomputes S^T and dP^T and accumulates dQ^T = K^T dS^T in registers, in a fixed order and
+//    without atomics, so dQ is bit-reproducible.
+//  * bwd_preprocess_kernel: delta = rowsum(O * dO), the reference's
+//    _backward_preprocess_do_o_dot (_triton_kernels_v2.py:532-608).
+#pragma once
+
+#include "fa2_common.cuh"
+
+namespace fa2 {
+
+struct BwdParams {
+  Tensor4 q, k, v, d_o, dq, dk, dv;
+  const float *lse;
+  const float *delta;
+  int batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded;
+  int n_tiles;  // key tiles (dK/dV kernel) or query tiles (dQ kernel)
+  float scale, scale_log2;
+  int vec;
+};
+
+struct PreParams {
+  Tensor4 o, d_o;
+  float *delta;
+  int batch, nheads, seqlen_q, headdim, seqlen_q_rounded;
+  int vec;
+};
+
+// ------------------------------------------------------------------------------------------
+// delta = rowsum(O * dO).  16 lanes per row, 16 rows per workgroup; rows in
+// [seqlen_q, seqlen_q_rounded) are written as zero.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_preprocess_kernel(const PreParams p) {
+  const int tid = threadIdx.x;
+  const int sub = tid & 15;
+  const int row = blockIdx.x * 16 + (tid >> 4);
+  const int bh = blockIdx.y;
+  const int b = bh / p.nheads, hd = bh % p.nheads;
+  const bool vec = p.vec != 0;
+  float acc = 0.f;
+  if (row < p.seqlen_q) {
+    const short *orow = (const short *)p.o.ptr + b * p.o.stride_batch + hd * p.o.stride_head +
+                        (int64_t)row * p.o.stride_seq;
+    const short *grow = (const short *)p.d_o.ptr + b * p.d_o.stride_batch +
+                        hd * p.d_o.stride_head + (int64_t)row * p.d_o.stride_seq;
+    for (int d0 = sub * 8; d0 < p.headdim; d0 += 128) {
+      s16x8 a = load_chunk(orow, d0, p.headdim, true, vec);
+      s16x8 g = load_chunk(grow, d0, p.headdim, true, vec);
+#pragma unroll
+      for (int j = 0; j < 8; j++) acc += Elem<T>::to_float(a[j]) * Elem<T>::to_float(g[j]);
+    }
+  }
+#pragma unroll
+  for (int off = 8; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 16);
+  if (sub == 0 && row < p.seqlen_q_rounded)
+    p.delta[(int64_t)bh * p.seqlen_q_rounded + row] = acc;
+}
+
+// ------------------------------------------------------------------------------------------
+// dQ kernel (query-tile parallel, fixed accumulation order).
+// ------------------------------------------------------------------------------------------
+constexpr int kDqWaves = 4;
+constexpr int kDqBlockQ = 32 * kDqWaves;
+
+template <int DP, int BKV>
+struct DqLayout {
+  static constexpr int KLD = DP + 8;
+  static constexpr int VLD = DP + 8;
+  static constexpr int K_ELEMS = BKV * KLD;
+  static constexpr int V_ELEMS = BKV * VLD;
+  static constexpr int STAGE_ELEMS = K_ELEMS + V_ELEMS;
+  static constexpr int PATCH_ELEMS = kDqWaves * 32 * (DP + 8);
+  static constexpr int TOTAL_ELEMS =
+      (2 * STAGE_ELEMS > PATCH_ELEMS) ? 2 * STAGE_ELEMS : PATCH_ELEMS;
+};
+
+template <typename T, int DP, int BKV>
+__global__ __launch_bounds__(64 * kDqWaves, (DP <= 96 ? 2 : 1)) void bwd_dq_kernel(const BwdParams p) {
+  using L = DqLayout<DP, BKV>;
+  constexpr int KS = DP / 16, DB = DP / 32, MB = BKV / 32, KS2 = BKV / 16, CPR = DP / 8;
+  constexpr int NTHREADS = 64 * kDqWaves;
+  constexpr int CPT = (BKV * CPR) / NTHREADS;
+  static_assert((BKV * CPR) % NTHREADS == 0, "tile must split evenly over the workgroup");
+
+  __shared__ __attribute__((aligned(16))) short smem[L::TOTAL_ELEMS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 31, h = lane >> 5;
+  const int i16 = lane & 15, g2 = (lane >> 4) & 1;
+
+  const int BH = p.batch * p.nheads;
+  const int bh = blockIdx.x % BH;
+  const int qt = p.n_tiles - 1 - blockIdx.x / BH;
+  const int b = bh / p.nheads, hd = bh % p.nheads;
+  const int q0 = qt * kDqBlockQ;
+  const int q0w = q0 + 32 * wave;
+  const bool vec = p.vec != 0;
+
+  const short *Q = (const short *)p.q.ptr + b * p.q.stride_batch + hd * p.q.stride_head;
+  const short *K = (const short *)p.k.ptr + b * p.k.stride_batch + hd * p.k.stride_head;
+  const short *V = (const short *)p.v.ptr + b * p.v.stride_batch + hd * p.v.stride_head;
+  const short *DO = (const short *)p.d_o.ptr + b * p.d_o.stride_batch + hd * p.d_o.stride_head;
+  short *DQ = (short *)p.dq.ptr + b * p.dq.stride_batch + hd * p.dq.stride_head;
+
+  // B operands: lane (c, h) holds row q0w + c of Q and of dO, columns 16 ks + 8 h + j.
+  s16x8 qf[KS], gf[KS];
+  float lse2 = 0.f, delta = 0.f;
+  {
+    const int row = q0w + c;
+    const bool ok = row < p.seqlen_q;
+    const short *qp = Q + (int64_t)row * p.q.stride_seq;
+    const short *gp = DO + (int64_t)row * p.d_o.stride_seq;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      qf[ks] = load_chunk(qp, 16 * ks + 8 * h, p.headdim, ok, vec);
+      gf[ks] = load_chunk(gp, 16 * ks + 8 * h, p.headdim, ok, vec);
+    }
+    if (ok) {
+      lse2 = p.lse[(int64_t)bh * p.seqlen_q_rounded + row] * kLog2e;
+      delta = p.delta[(int64_t)bh * p.seqlen_q_rounded + row];
+    }
+  }
+
+  const int kv_end = min(q0 + kDqBlockQ, p.seqlen_k);
+  const int n_tiles = (kv_end + BKV - 1) / BKV;
+
+  s16x8 kreg[CPT], vreg[CPT];
+  auto load_tile = [&](int kvt) {
+#pragma unroll
+    for (int i = 0; i < CPT; i++) {
+      const int id = tid + NTHREADS * i;
+      const int r = id / CPR, cc = id % CPR;
+      const int kv = kvt + r;
+      const bool ok = kv < p.seqlen_k;
+      kreg[i] = load_chunk(K + (int64_t)kv * p.k.stride_seq, cc * 8, p.headdim, ok, vec);
+      vreg[i] = load_chunk(V + (int64_t)kv * p.v.stride_seq, cc * 8, p.headdim, ok, vec);
+    }
+  };
+  auto store_tile = [&](int buf) {
+    short *sk = smem + buf * L::STAGE_ELEMS;
+    short *sv = sk + L::K_ELEMS;
+#pragma unroll
+    for (int i = 0; i < CPT; i++) {
+      const int id = tid + NTHREADS * i;
+      const int r = id / CPR, cc = id % CPR;
+      *reinterpret_cast<s16x8 *>(sk + r * L::KLD + cc * 8) = kreg[i];
+      *reinterpret_cast<s16x8 *>(sv + r * L::VLD + cc * 8) = vreg[i];
+    }
+  };
+
+  f32x16 dqacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) dqacc[db][i] = 0.f;
+
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+
+  const int row_frag_off = c * L::KLD + 8 * h;  // KLD == VLD
+  const int tr_frag_off = (4 * h + (i16 >> 2)) * L::KLD + 16 * g2 + 4 * (i16 & 3);
+  static_assert(L::KLD == L::VLD, "shared fragment offsets assume equal pitches");
+
+  for (int t = 0; t < n_tiles; t++) {
+    const int buf = t & 1;
+    const int kvt = t * BKV;
+    const bool more = (t + 1) < n_tiles;
+    if (more) load_tile(kvt + BKV);
+
+    int nact = (q0w + 31 - kvt) / 32 + 1;
+    nact = (q0w + 31 < kvt) ? 0 : min(nact, MB);
+
+    if (nact > 0) {
+      const short *sk = smem + buf * L::STAGE_ELEMS;
+      const short *sv = sk + L::K_ELEMS;
+      const bool need_mask = (kvt + 32 * nact - 1 > q0w) || (kvt + 32 * nact > p.seqlen_k);
+      const int qrow = q0w + c;
+
+      s16x8 dsf[KS2];
+#pragma unroll
+      for (int mb = 0; mb < MB; mb++) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          s[i] = 0.f;
+          dp[i] = 0.f;
+        }
+        if (mb < nact) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ks++) {
+            s16x8 a = *reinterpret_cast<const s16x8 *>(sk + row_frag_off + 32 * mb * L::KLD + 16 * ks);
+            s = Elem<T>::mfma(a, qf[ks], s);
+          }
+#pragma unroll
+          for (int ks = 0; ks < KS; ks++) {
+            s16x8 a = *reinterpret_cast<const s16x8 *>(sv + row_frag_off + 32 * mb * L::VLD + 16 * ks);
+            dp = Elem<T>::mfma(a, gf[ks], dp);
+          }
+        }
+        f32x16 ds;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          float pr = fast_exp2(s[i] * p.scale_log2 - lse2);
+          if (need_mask) {
+            const int kv = kvt + 32 * mb + 8 * (i >> 2) + 4 * h + (i & 3);
+            if (kv > qrow || kv >= p.seqlen_k) pr = 0.f;
+          }
+          ds[i] = pr * (dp[i] - delta);
+        }
+        if (mb >= nact) {
+#pragma unroll
+          for (int i = 0; i < 16; i++) ds[i] = 0.f;
+        }
+        f32x8 lo = {ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]};
+        f32x8 hi = {ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]};
+        dsf[2 * mb] = Elem<T>::pack8(lo);
+        dsf[2 * mb + 1] = Elem<T>::pack8(hi);
+      }
+
+#pragma unroll
+      for (int ks2 = 0; ks2 < KS2; ks2++) {
+        if ((ks2 >> 1) < nact) {
+#pragma unroll
+          for (int db = 0; db < DB; db++) {
+            s16x8 a = lds_read_tr_frag(sk + tr_frag_off + 16 * ks2 * L::KLD + 32 * db, L::KLD);
+            dqacc[db] = Elem<T>::mfma(a, dsf[ks2], dqacc[db]);
+          }
+        }
+      }
+    }
+
+    if (more) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  short *patch = smem + wave * 32 * (DP + 8);
+  store_transposed_acc<T, DP>(dqacc, p.scale, patch, DQ + (int64_t)q0w * p.dq.stride_seq,
+                              p.dq.stride_seq, p.seqlen_q - q0w, p.headdim, vec);
+}
+
+// ------------------------------------------------------------------------------------------
+// dK/dV kernel (key-tile parallel).
+// ------------------------------------------------------------------------------------------
+constexpr int kDkvWaves = 4;
+constexpr int kDkvBlockKV = 32 * kDkvWaves;
+
+template <int DP, int BQ>
+struct DkvLayout {
+  static constexpr int QLD = DP + 8;
+  static constexpr int Q_ELEMS = BQ * QLD;
+  // One stage: Q tile, dO tile, then lse*log2e and delta as floats (2 shorts each).
+  static constexpr int STAGE_ELEMS = 2 * Q_ELEMS + 4 * BQ;
+  static constexpr int PATCH_ELEMS = kDkvWaves * 32 * (DP + 8);
+  static constexpr int TOTAL_ELEMS =
+      (2 * STAGE_ELEMS > PATCH_ELEMS) ? 2 * STAGE_ELEMS : PATCH_ELEMS;
+};
+
+template <typename T, int DP, int BQ>
+__global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdParams p) {
+  using L = DkvLayout<DP, BQ>;
+  constexpr int KS = DP / 16, DB = DP / 32, MQ = BQ / 32, CPR = DP / 8;
+  constexpr int NTHREADS = 64 * kDkvWaves;
+  constexpr int CPT = (BQ * CPR) / NTHREADS;
+  static_assert((BQ * CPR) % NTHREADS == 0, "tile must split evenly over the workgroup");
+  static_assert(BQ <= NTHREADS, "one thread per row loads lse and delta");
+
+  __shared__ __attribute__((aligned(16))) short smem[L::TOTAL_ELEMS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 31, h = lane >> 5;
+  const int i16 = lane & 15, g2 = (lane >> 4) & 1;
+
+  // Key tile 0 has the longest query range: issue tiles in ascending order (heaviest first).
+  const int BH = p.batch * p.nheads;
+  const int bh = blockIdx.x % BH;
+  const int kt = blockIdx.x / BH;
+  const int b = bh / p.nheads, hd = bh % p.nheads;
+  const int kv0 = kt * kDkvBlockKV;
+  const int kv0w = kv0 + 32 * wave;
+  const bool vec = p.vec != 0;
+
+  const short *Q = (const short *)p.q.ptr + b * p.q.stride_batch + hd * p.q.stride_head;
+  const short *K = (const short *)p.k.ptr + b * p.k.stride_batch + hd * p.k.stride_head;
+  const short *V = (const short *)p.v.ptr + b * p.v.stride_batch + hd * p.v.stride_head;
+  const short *DO = (const short *)p.d_o.ptr + b * p.d_o.stride_batch + hd * p.d_o.stride_head;
+  short *DK = (short *)p.dk.ptr + b * p.dk.stride_batch + hd * p.dk.stride_head;
+  short *DV = (short *)p.dv.ptr + b * p.dv.stride_batch + hd * p.dv.stride_head;
+  const float *LSE = p.lse + (int64_t)bh * p.seqlen_q_rounded;
+  const float *DELTA = p.delta + (int64_t)bh * p.seqlen_q_rounded;
+
+  // B operands: lane (c, h) holds row kv0w + c of K and of V, columns 16 ks + 8 h + j.
+  s16x8 kf[KS], vf[KS];
+  {
+    const int row = kv0w + c;
+    const bool ok = row < p.seqlen_k;
+    const short *kp = K + (int64_t)row * p.k.stride_seq;
+    const short *vp = V + (int64_t)row * p.v.stride_seq;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      kf[ks] = load_chunk(kp, 16 * ks + 8 * h, p.headdim, ok, vec);
+      vf[ks] = load_chunk(vp, 16 * ks + 8 * h, p.headdim, ok, vec);
+    }
+  }
+
+  // First query tile that can see this key tile (row >= col), aligned down to BQ.
+  const int q_begin = (kv0 / BQ) * BQ;
+  const int n_tiles = (p.seqlen_q > q_begin) ? (p.seqlen_q - q_begin + BQ - 1) / BQ : 0;
+
+  s16x8 qreg[CPT], greg[CPT];
+  float lse_reg = 0.f, delta_reg = 0.f;
+  auto load_tile = [&](int qt0) {
+#pragma unroll
+    for (int i = 0; i < CPT; i++) {
+      const int id = tid + NTHREADS * i;
+      const int r = id / CPR, cc = id % CPR;
+      const int row = qt0 + r;
+      const bool ok = row < p.seqlen_q;
+      qreg[i] = load_chunk(Q + (int64_t)row * p.q.stride_seq, cc * 8, p.headdim, ok, vec);
+      greg[i] = load_chunk(DO + (int64_t)row * p.d_o.stride_seq, cc * 8, p.headdim, ok, vec);
+    }
+    if (tid < BQ) {
+      const int row = qt0 + tid;
+      const bool ok = row < p.seqlen_q;
+      lse_reg = ok ? LSE[row] * kLog2e : 0.f;
+      delta_reg = ok ? DELTA[row] : 0.f;
+    }
+  };
+  auto store_tile = [&](int buf) {
+    short *sq = smem + buf * L::STAGE_ELEMS;
+    short *sg = sq + L::Q_ELEMS;
+    float *sl = reinterpret_cast<float *>(sg + L::Q_ELEMS);
+#pragma unroll
+    for (int i = 0; i < CPT; i++) {
+      const int id = tid + NTHREADS * i;
+      const int r = id / CPR, cc = id % CPR;
+      *reinterpret_cast<s16x8 *>(sq + r * L::QLD + cc * 8) = qreg[i];
+      *reinterpret_cast<s16x8 *>(sg + r * L::QLD + cc * 8) = greg[i];
+    }
+    if (tid < BQ) {
+      sl[tid] = lse_reg;
+      sl[BQ + tid] = delta_reg;
+    }
+  };
+
+  f32x16 dkacc[DB], dvacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      dkacc[db][i] = 0.f;
+      dvacc[db][i] = 0.f;
+    }
+
+  if (n_tiles > 0) {
+    load_tile(q_begin);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  const int row_frag_off = c * L::QLD + 8 * h;
+  const int tr_frag_off = (4 * h + (i16 >> 2)) * L::QLD + 16 * g2 + 4 * (i16 & 3);
+  const int kvcol = kv0w + c;
+
+  for (int t = 0; t < n_tiles; t++) {
+    const int buf = t & 1;
+    const int qt0 = q_begin + t * BQ;
+    const bool more = (t + 1) < n_tiles;
+    if (more) load_tile(qt0 + BQ);
+
+    const short *sq = smem + buf * L::STAGE_ELEMS;
+    const short *sg = sq + L::Q_ELEMS;
+    const float *sl = reinterpret_cast<const float *>(sg + L::Q_ELEMS);
+
+#pragma unroll
+    for (int mq = 0; mq < MQ; mq++) {
+      const int qb = qt0 + 32 * mq;  // first query row of this 32-row block
+      // Skip blocks whose every row lies above this wave's first key column.
+      if (qb + 31 >= kv0w) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          s[i] = 0.f;
+          dp[i] = 0.f;
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          s16x8 a = *reinterpret_cast<const s16x8 *>(sq + row_frag_off + 32 * mq * L::QLD + 16 * ks);
+          s = Elem<T>::mfma(a, kf[ks], s);
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          s16x8 a = *reinterpret_cast<const s16x8 *>(sg + row_frag_off + 32 * mq * L::QLD + 16 * ks);
+          dp = Elem<T>::mfma(a, vf[ks], dp);
+        }
+        const bool need_mask = (qb < kv0w + 31);
+        f32x16 pr, ds;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const f32x4 l4 = *reinterpret_cast<const f32x4 *>(sl + 32 * mq + 8 * g + 4 * h);
+          const f32x4 d4 = *reinterpret_cast<const f32x4 *>(sl + BQ + 32 * mq + 8 * g + 4 * h);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int i = 4 * g + e;
+            float x = fast_exp2(s[i] * p.scale_log2 - l4[e]);
+            if (need_mask) {
+              const int qrow = qb + 8 * g + 4 * h + e;
+              if (kvcol > qrow) x = 0.f;
+            }
+            pr[i] = x;
+            ds[i] = x * (dp[i] - d4[e]);
+          }
+        }
+        f32x8 plo = {pr[0], pr[1], pr[2], pr[3], pr[4], pr[5], pr[6], pr[7]};
+        f32x8 phi = {pr[8], pr[9], pr[10], pr[11], pr[12], pr[13], pr[14], pr[15]};
+        f32x8 dlo = {ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]};
+        f32x8 dhi = {ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]};
+        s16x8 pf[2] = {Elem<T>::pack8(plo), Elem<T>::pack8(phi)};
+        s16x8 dsf[2] = {Elem<T>::pack8(dlo), Elem<T>::pack8(dhi)};
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+#pragma unroll
+          for (int db = 0; db < DB; db++) {
+            const int off = tr_frag_off + (32 * mq + 16 * tt) * L::QLD + 32 * db;
+            s16x8 ag = lds_read_tr_frag(sg + off, L::QLD);
+            dvacc[db] = Elem<T>::mfma(ag, pf[tt], dvacc[db]);
+            s16x8 aq = lds_read_tr_frag(sq + off, L::QLD);
+            dkacc[db] = Elem<T>::mfma(aq, dsf[tt], dkacc[db]);
+          }
+        }
+      }
+    }
+
+    if (more) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  short *patch = smem + wave * 32 * (DP + 8);
+  store_transposed_acc<T, DP>(dvacc, 1.0f, patch, DV + (int64_t)kv0w * p.dv.stride_seq,
+                              p.dv.stride_seq, p.seqlen_k - kv0w, p.headdim, vec);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  store_transposed_acc<T, DP>(dkacc, p.scale, patch, DK + (int64_t)kv0w * p.dk.stride_seq,
+                              p.dk.stride_seq, p.seqlen_k - kv0w, p.headdim, vec);
+}
+
+}  // namespace fa2

@@ -1,0 +1,341 @@
+// C ABI of libfa2_gfx950.so: argument validation, the gfx950 tile table and kernel launches.
+// Declarations and the reference interfaces they replace are in include/fa2_gfx950.h.
+
+#include "fa2_gfx950.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+
+#include "fa2_bwd.cuh"
+#include "fa2_fwd.cuh"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int status, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+// ---- gfx950 tile/wave table -----------------------------------------------------------------
+// One row per padded head dimension.  All rows use 4 waves of 64 lanes per workgroup and the
+// 32x32x16 MFMA; a wave always owns 32 sequence positions of the operand it keeps in registers.
+constexpr int kFwdBlockKV = 64;
+constexpr int kDqBlockKV = 64;
+constexpr int kDkvBlockQ = 64;
+
+const fa2_config_info kTable[] = {
+    // id  DP   fwd: BQ   BKV waves   dK/dV: BQ  BKV  waves   dQ: BQ  BKV  waves
+    {0, 32, fa2::kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, fa2::kDkvBlockKV, 4, fa2::kDqBlockQ, kDqBlockKV, 4},
+    {1, 64, fa2::kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, fa2::kDkvBlockKV, 4, fa2::kDqBlockQ, kDqBlockKV, 4},
+    {2, 96, fa2::kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, fa2::kDkvBlockKV, 4, fa2::kDqBlockQ, kDqBlockKV, 4},
+    {3, 128, fa2::kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, fa2::kDkvBlockKV, 4, fa2::kDqBlockQ, kDqBlockKV, 4},
+};
+constexpr int kTableRows = sizeof(kTable) / sizeof(kTable[0]);
+
+int pick_config(int headdim) {
+  for (int i = 0; i < kTableRows; i++)
+    if (headdim <= kTable[i].headdim_padded) return i;
+  return -1;
+}
+
+int resolve_config(int config_id, int headdim, int *out) {
+  if (config_id == FA2_CONFIG_AUTO) {
+    *out = pick_config(headdim);
+    return FA2_OK;
+  }
+  if (config_id < 0 || config_id >= kTableRows)
+    return fail(FA2_ERR_BAD_CONFIG, "config id %d outside the table [0, %d)", config_id, kTableRows);
+  if (kTable[config_id].headdim_padded < headdim)
+    return fail(FA2_ERR_BAD_CONFIG, "config %d is built for headdim <= %d, got %d", config_id,
+                kTable[config_id].headdim_padded, headdim);
+  *out = config_id;
+  return FA2_OK;
+}
+
+int check_common(int batch, int nheads, int seqlen_q, int seqlen_k, int headdim,
+                 int seqlen_q_rounded, int dtype) {
+  if (batch <= 0 || nheads <= 0 || seqlen_q <= 0 || seqlen_k <= 0 || headdim <= 0)
+    return fail(FA2_ERR_BAD_SHAPE, "sizes must be positive: batch=%d nheads=%d seqlen_q=%d seqlen_k=%d headdim=%d",
+                batch, nheads, seqlen_q, seqlen_k, headdim);
+  if (seqlen_q_rounded < seqlen_q)
+    return fail(FA2_ERR_BAD_SHAPE, "seqlen_q_rounded=%d < seqlen_q=%d", seqlen_q_rounded, seqlen_q);
+  if (headdim > FA2_MAX_HEADDIM)
+    return fail(FA2_ERR_HEADDIM, "Supports head dimensions only up to %d, got %d", FA2_MAX_HEADDIM, headdim);
+  if (dtype != FA2_DTYPE_F16 && dtype != FA2_DTYPE_BF16)
+    return fail(FA2_ERR_BAD_DTYPE, "dtype %d is neither FA2_DTYPE_F16 nor FA2_DTYPE_BF16", dtype);
+  if ((int64_t)batch * nheads > 0x7fffffff / 64)
+    return fail(FA2_ERR_TOO_LARGE, "batch*nheads=%lld too large", (long long)batch * nheads);
+  return FA2_OK;
+}
+
+int check_tensor(const char *name, const fa2::Tensor4 &t) {
+  if (t.ptr == nullptr) return fail(FA2_ERR_NULL_POINTER, "%s is NULL", name);
+  if (t.stride_batch < 0 || t.stride_head < 0 || t.stride_seq < 0)
+    return fail(FA2_ERR_BAD_STRIDE, "%s has a negative stride", name);
+  return FA2_OK;
+}
+
+// 16-byte accesses need headdim % 8 == 0, 16-byte aligned bases and strides that keep rows aligned.
+bool vec_ok(const fa2::Tensor4 &t, int headdim) {
+  return headdim % 8 == 0 && (reinterpret_cast<uintptr_t>(t.ptr) % 16 == 0) &&
+         t.stride_batch % 8 == 0 && t.stride_head % 8 == 0 && t.stride_seq % 8 == 0;
+}
+
+fa2::Tensor4 tensor(const void *ptr, int64_t sb, int64_t sh, int64_t ss) {
+  return fa2::Tensor4{const_cast<void *>(ptr), sb, sh, ss};
+}
+
+int launch_status(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(FA2_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return FA2_OK;
+}
+
+template <typename T>
+void launch_fwd(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
+  dim3 block(64 * fa2::kFwdWaves);
+  switch (dp) {
+    case 32: hipLaunchKernelGGL((fa2::fwd_kernel<T, 32, kFwdBlockKV>), grid, block, 0, s, p); break;
+    case 64: hipLaunchKernelGGL((fa2::fwd_kernel<T, 64, kFwdBlockKV>), grid, block, 0, s, p); break;
+    case 96: hipLaunchKernelGGL((fa2::fwd_kernel<T, 96, kFwdBlockKV>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fa2::fwd_kernel<T, 128, kFwdBlockKV>), grid, block, 0, s, p); break;
+  }
+}
+
+template <typename T>
+void launch_dq(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
+  dim3 block(64 * fa2::kDqWaves);
+  switch (dp) {
+    case 32: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 32, kDqBlockKV>), grid, block, 0, s, p); break;
+    case 64: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 64, kDqBlockKV>), grid, block, 0, s, p); break;
+    case 96: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 96, kDqBlockKV>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 128, kDqBlockKV>), grid, block, 0, s, p); break;
+  }
+}
+
+template <typename T>
+void launch_dkdv(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
+  dim3 block(64 * fa2::kDkvWaves);
+  switch (dp) {
+    case 32: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 32, kDkvBlockQ>), grid, block, 0, s, p); break;
+    case 64: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 64, kDkvBlockQ>), grid, block, 0, s, p); break;
+    case 96: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 96, kDkvBlockQ>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 128, kDkvBlockQ>), grid, block, 0, s, p); break;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int fa2_abi_version(void) { return FA2_ABI_VERSION; }
+
+const char *fa2_last_error_string(void) { return g_error; }
+
+const char *fa2_status_string(int status) {
+  switch (status) {
+    case FA2_OK: return "FA2_OK";
+    case FA2_ERR_NULL_POINTER: return "FA2_ERR_NULL_POINTER";
+    case FA2_ERR_BAD_SHAPE: return "FA2_ERR_BAD_SHAPE";
+    case FA2_ERR_BAD_DTYPE: return "FA2_ERR_BAD_DTYPE";
+    case FA2_ERR_HEADDIM: return "FA2_ERR_HEADDIM";
+    case FA2_ERR_BAD_STRIDE: return "FA2_ERR_BAD_STRIDE";
+    case FA2_ERR_BAD_CONFIG: return "FA2_ERR_BAD_CONFIG";
+    case FA2_ERR_WORKSPACE: return "FA2_ERR_WORKSPACE";
+    case FA2_ERR_LAUNCH: return "FA2_ERR_LAUNCH";
+    case FA2_ERR_TOO_LARGE: return "FA2_ERR_TOO_LARGE";
+    default: return "FA2_ERR_UNKNOWN";
+  }
+}
+
+int fa2_config_count(void) { return kTableRows; }
+
+int fa2_config_get(int config_id, fa2_config_info *out) {
+  if (out == nullptr) return fail(FA2_ERR_NULL_POINTER, "out is NULL");
+  if (config_id < 0 || config_id >= kTableRows)
+    return fail(FA2_ERR_BAD_CONFIG, "config id %d outside the table [0, %d)", config_id, kTableRows);
+  *out = kTable[config_id];
+  return FA2_OK;
+}
+
+int fa2_pick_config(int dtype, int headdim, int seqlen_q, int seqlen_k, int deterministic) {
+  (void)deterministic;
+  if (dtype != FA2_DTYPE_F16 && dtype != FA2_DTYPE_BF16)
+    return -fail(FA2_ERR_BAD_DTYPE, "dtype %d is neither FA2_DTYPE_F16 nor FA2_DTYPE_BF16", dtype);
+  if (headdim <= 0 || seqlen_q <= 0 || seqlen_k <= 0)
+    return -fail(FA2_ERR_BAD_SHAPE, "sizes must be positive: headdim=%d seqlen_q=%d seqlen_k=%d",
+                 headdim, seqlen_q, seqlen_k);
+  int id = pick_config(headdim);
+  if (id < 0)
+    return -fail(FA2_ERR_HEADDIM, "Supports head dimensions only up to %d, got %d", FA2_MAX_HEADDIM, headdim);
+  return id;
+}
+
+int fa2_fwd(const void *q, const void *k, const void *v, void *o, float *lse, int batch, int nheads,
+            int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded, int64_t q_sb,
+            int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb,
+            int64_t v_sh, int64_t v_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss,
+            float softmax_scale, int dtype, int config_id, void *stream) {
+  int rc = check_common(batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded, dtype);
+  if (rc) return rc;
+  fa2::FwdParams p;
+  p.q = tensor(q, q_sb, q_sh, q_ss);
+  p.k = tensor(k, k_sb, k_sh, k_ss);
+  p.v = tensor(v, v_sb, v_sh, v_ss);
+  p.o = tensor(o, o_sb, o_sh, o_ss);
+  if ((rc = check_tensor("q", p.q)) || (rc = check_tensor("k", p.k)) ||
+      (rc = check_tensor("v", p.v)) || (rc = check_tensor("o", p.o)))
+    return rc;
+  if (lse == nullptr) return fail(FA2_ERR_NULL_POINTER, "lse is NULL");
+  if (!(softmax_scale > 0.f) || !std::isfinite(softmax_scale))
+    return fail(FA2_ERR_BAD_SHAPE, "softmax_scale must be positive and finite, got %g", (double)softmax_scale);
+  int cfg;
+  if ((rc = resolve_config(config_id, headdim, &cfg))) return rc;
+
+  p.lse = lse;
+  p.batch = batch;
+  p.nheads = nheads;
+  p.seqlen_q = seqlen_q;
+  p.seqlen_k = seqlen_k;
+  p.headdim = headdim;
+  p.seqlen_q_rounded = seqlen_q_rounded;
+  p.n_qtiles = (seqlen_q + fa2::kFwdBlockQ - 1) / fa2::kFwdBlockQ;
+  p.scale = softmax_scale;
+  p.scale_log2 = softmax_scale * fa2::kLog2e;
+  p.vec = vec_ok(p.q, headdim) && vec_ok(p.k, headdim) && vec_ok(p.v, headdim) && vec_ok(p.o, headdim);
+
+  const int64_t nwg = (int64_t)p.n_qtiles * batch * nheads;
+  if (nwg > 0x7fffffff) return fail(FA2_ERR_TOO_LARGE, "grid of %lld workgroups too large", (long long)nwg);
+  dim3 grid((unsigned)nwg);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int dp = kTable[cfg].headdim_padded;
+  if (dtype == FA2_DTYPE_BF16)
+    launch_fwd<__bf16>(dp, p, grid, s);
+  else
+    launch_fwd<_Float16>(dp, p, grid, s);
+  return launch_status("fa2_fwd launch");
+}
+
+int fa2_bwd_preprocess(const void *o, const void *d_o, float *delta, int batch, int nheads,
+                       int seqlen_q, int headdim, int seqlen_q_rounded, int64_t o_sb, int64_t o_sh,
+                       int64_t o_ss, int64_t do_sb, int64_t do_sh, int64_t do_ss, int dtype,
+                       void *stream) {
+  int rc = check_common(batch, nheads, seqlen_q, 1, headdim, seqlen_q_rounded, dtype);
+  if (rc) return rc;
+  fa2::PreParams p;
+  p.o = tensor(o, o_sb, o_sh, o_ss);
+  p.d_o = tensor(d_o, do_sb, do_sh, do_ss);
+  if ((rc = check_tensor("o", p.o)) || (rc = check_tensor("d_o", p.d_o))) return rc;
+  if (delta == nullptr) return fail(FA2_ERR_NULL_POINTER, "delta is NULL");
+  p.delta = delta;
+  p.batch = batch;
+  p.nheads = nheads;
+  p.seqlen_q = seqlen_q;
+  p.headdim = headdim;
+  p.seqlen_q_rounded = seqlen_q_rounded;
+  p.vec = vec_ok(p.o, headdim) && vec_ok(p.d_o, headdim);
+  const int64_t bh = (int64_t)batch * nheads;
+  if (bh > 65535) return fail(FA2_ERR_TOO_LARGE, "batch*nheads=%lld exceeds the grid's second dimension", (long long)bh);
+  dim3 grid((seqlen_q_rounded + 15) / 16, (unsigned)bh);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == FA2_DTYPE_BF16)
+    hipLaunchKernelGGL((fa2::bwd_preprocess_kernel<__bf16>), grid, dim3(256), 0, s, p);
+  else
+    hipLaunchKernelGGL((fa2::bwd_preprocess_kernel<_Float16>), grid, dim3(256), 0, s, p);
+  return launch_status("fa2_bwd_preprocess launch");
+}
+
+size_t fa2_bwd_workspace_bytes(int batch, int nheads, int seqlen_q, int seqlen_k, int headdim,
+                               int deterministic, int config_id) {
+  (void)batch; (void)nheads; (void)seqlen_q; (void)seqlen_k; (void)headdim;
+  (void)deterministic; (void)config_id;
+  // Both modes currently write dQ exactly once from registers: no accumulation buffer.
+  return 0;
+}
+
+int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const float *lse,
+            const float *delta, void *workspace, void *dq, void *dk, void *dv, int batch,
+            int nheads, int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded, int64_t q_sb,
+            int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb,
+            int64_t v_sh, int64_t v_ss, int64_t do_sb, int64_t do_sh, int64_t do_ss, int64_t dq_sb,
+            int64_t dq_sh, int64_t dq_ss, int64_t dk_sb, int64_t dk_sh, int64_t dk_ss,
+            int64_t dv_sb, int64_t dv_sh, int64_t dv_ss, float softmax_scale, int dtype,
+            int deterministic, int config_id, void *stream) {
+  (void)workspace;
+  (void)deterministic;
+  int rc = check_common(batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded, dtype);
+  if (rc) return rc;
+  fa2::BwdParams p;
+  p.q = tensor(q, q_sb, q_sh, q_ss);
+  p.k = tensor(k, k_sb, k_sh, k_ss);
+  p.v = tensor(v, v_sb, v_sh, v_ss);
+  p.d_o = tensor(d_o, do_sb, do_sh, do_ss);
+  p.dq = tensor(dq, dq_sb, dq_sh, dq_ss);
+  p.dk = tensor(dk, dk_sb, dk_sh, dk_ss);
+  p.dv = tensor(dv, dv_sb, dv_sh, dv_ss);
+  if ((rc = check_tensor("q", p.q)) || (rc = check_tensor("k", p.k)) ||
+      (rc = check_tensor("v", p.v)) || (rc = check_tensor("d_o", p.d_o)) ||
+      (rc = check_tensor("dq", p.dq)) || (rc = check_tensor("dk", p.dk)) ||
+      (rc = check_tensor("dv", p.dv)))
+    return rc;
+  if (lse == nullptr) return fail(FA2_ERR_NULL_POINTER, "lse is NULL");
+  if (delta == nullptr) return fail(FA2_ERR_NULL_POINTER, "delta is NULL");
+  if (!(softmax_scale > 0.f) || !std::isfinite(softmax_scale))
+    return fail(FA2_ERR_BAD_SHAPE, "softmax_scale must be positive and finite, got %g", (double)softmax_scale);
+  int cfg;
+  if ((rc = resolve_config(config_id, headdim, &cfg))) return rc;
+
+  p.lse = lse;
+  p.delta = delta;
+  p.batch = batch;
+  p.nheads = nheads;
+  p.seqlen_q = seqlen_q;
+  p.seqlen_k = seqlen_k;
+  p.headdim = headdim;
+  p.seqlen_q_rounded = seqlen_q_rounded;
+  p.scale = softmax_scale;
+  p.scale_log2 = softmax_scale * fa2::kLog2e;
+  p.vec = vec_ok(p.q, headdim) && vec_ok(p.k, headdim) && vec_ok(p.v, headdim) &&
+          vec_ok(p.d_o, headdim) && vec_ok(p.dq, headdim) && vec_ok(p.dk, headdim) &&
+          vec_ok(p.dv, headdim);
+
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int dp = kTable[cfg].headdim_padded;
+  const int64_t bh = (int64_t)batch * nheads;
+
+  {  // dK, dV
+    fa2::BwdParams pk = p;
+    pk.n_tiles = (seqlen_k + fa2::kDkvBlockKV - 1) / fa2::kDkvBlockKV;
+    const int64_t nwg = pk.n_tiles * bh;
+    if (nwg > 0x7fffffff) return fail(FA2_ERR_TOO_LARGE, "grid of %lld workgroups too large", (long long)nwg);
+    dim3 grid((unsigned)nwg);
+    if (dtype == FA2_DTYPE_BF16)
+      launch_dkdv<__bf16>(dp, pk, grid, s);
+    else
+      launch_dkdv<_Float16>(dp, pk, grid, s);
+    if ((rc = launch_status("fa2_bwd dK/dV launch"))) return rc;
+  }
+  {  // dQ
+    fa2::BwdParams pq = p;
+    pq.n_tiles = (seqlen_q + fa2::kDqBlockQ - 1) / fa2::kDqBlockQ;
+    const int64_t nwg = pq.n_tiles * bh;
+    if (nwg > 0x7fffffff) return fail(FA2_ERR_TOO_LARGE, "grid of %lld workgroups too large", (long long)nwg);
+    dim3 grid((unsigned)nwg);
+    if (dtype == FA2_DTYPE_BF16)
+      launch_dq<__bf16>(dp, pq, grid, s);
+    else
+      launch_dq<_Float16>(dp, pq, grid, s);
+    if ((rc = launch_status("fa2_bwd dQ launch"))) return rc;
+  }
+  return FA2_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,179 @@
+// Shared device helpers for the gfx950 FlashAttention-2 kernels.
+//
+// Everything here is written for CDNA4 wave64 and the v_mfma_f32_32x32x16_{bf16,f16}
+// instruction.  Register layouts of that instruction (lane = 32*h + c, h in {0,1}, c in 0..31):
+//   A operand (32 x 16):  lane holds A[m = c][k = 8h + j],            j = 0..7
+//   B operand (16 x 32):  lane holds B[k = 8h + j][n = c],            j = 0..7
+//   C/D       (32 x 32):  lane holds C[m = 8*(i/4) + 4h + i%4][n = c], i = 0..15
+// The k index is only a summation label, so any consistent assignment of the 8 values per lane
+// works as long as A and B agree.  The kernels exploit this: an accumulator tile re-enters the
+// next MFMA as a B operand straight from registers, with
+//   element j of lane (c, h)  <->  row 16*t + 8*(j/4) + 4h + j%4   (t = which half of the 32 rows)
+// and the matching A operand is fetched from row-major LDS tiles with ds_read_b64_tr_b16, the
+// transposing LDS read of gfx950: within each group of 16 lanes, lane i receives elements
+// e = 0..3 taken from lane (4e + i/4)'s 64-bit word, position i%4.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa2 {
+
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// One (batch, nheads, seqlen, headdim) tensor: base pointer and strides in elements.
+struct Tensor4 {
+  void *ptr;
+  int64_t stride_batch, stride_head, stride_seq;
+};
+
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<__bf16> {
+  static __device__ __forceinline__ f32x16 mfma(s16x8 a, s16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ s16x8 pack8(f32x8 x) {
+    return __builtin_bit_cast(s16x8, __builtin_convertvector(x, bf16x8));
+  }
+  static __device__ __forceinline__ s16x4 pack4(f32x4 x) {
+    return __builtin_bit_cast(s16x4, __builtin_convertvector(x, bf16x4));
+  }
+  static __device__ __forceinline__ float to_float(short x) {
+    return __builtin_bit_cast(float, ((unsigned)(unsigned short)x) << 16);
+  }
+};
+
+template <>
+struct Elem<_Float16> {
+  static __device__ __forceinline__ f32x16 mfma(s16x8 a, s16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ s16x8 pack8(f32x8 x) {
+    return __builtin_bit_cast(s16x8, __builtin_convertvector(x, f16x8));
+  }
+  static __device__ __forceinline__ s16x4 pack4(f32x4 x) {
+    return __builtin_bit_cast(s16x4, __builtin_convertvector(x, f16x4));
+  }
+  static __device__ __forceinline__ float to_float(short x) {
+    return (float)__builtin_bit_cast(_Float16, x);
+  }
+};
+
+// Transposing 64-bit LDS read (ds_read_b64_tr_b16).
+__device__ __forceinline__ s16x4 lds_read_tr(const short *p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p));
+}
+
+// A-operand fragment whose k index runs along the ROWS of a row-major LDS tile: two transposing
+// reads, rows r0..r0+3 and r0+8..r0+11 as seen by this lane group.  `p` already points at this
+// lane's (row, column) for the first read; `ld` is the tile's row pitch in elements.
+__device__ __forceinline__ s16x8 lds_read_tr_frag(const short *p, int ld) {
+  s16x4 lo = lds_read_tr(p);
+  s16x4 hi = lds_read_tr(p + 8 * ld);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Exchange between lane l and lane l^32 with v_permlane32_swap.  With both operands equal to x
+// the instruction returns (x[l], x[l+32]) in lanes < 32 and (x[l-32], x[l]) in lanes >= 32.
+// The two results are copied to scalars before any bit cast: __builtin_bit_cast applied directly
+// to an element of the returned vector reads element 0 with this compiler.
+struct HalfPair {
+  float lo, hi;
+};
+__device__ __forceinline__ HalfPair both_halves(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned a = r[0], b = r[1];
+  return HalfPair{__builtin_bit_cast(float, a), __builtin_bit_cast(float, b)};
+}
+__device__ __forceinline__ float max_over_halves(float x) {
+  const HalfPair p = both_halves(x);
+  return fmaxf(p.lo, p.hi);
+}
+__device__ __forceinline__ float sum_over_halves(float x) {
+  const HalfPair p = both_halves(x);
+  return p.lo + p.hi;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Load 8 consecutive 16-bit elements row[d0 .. d0+7], zero beyond `headdim` or when the row is
+// out of range.  `vec` (uniform) says 16-byte loads are legal: headdim % 8 == 0 and every row
+// start is 16-byte aligned.
+__device__ __forceinline__ s16x8 load_chunk(const short *row, int d0, int headdim, bool row_ok,
+                                            bool vec) {
+  s16x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (!row_ok) return r;
+  if (vec) {
+    if (d0 < headdim) r = *reinterpret_cast<const s16x8 *>(row + d0);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (d0 + j < headdim) r[j] = row[d0 + j];
+  }
+  return r;
+}
+
+__device__ __forceinline__ void store_chunk(short *row, int d0, int headdim, bool row_ok, bool vec,
+                                            s16x8 v) {
+  if (!row_ok) return;
+  if (vec) {
+    if (d0 < headdim) *reinterpret_cast<s16x8 *>(row + d0) = v;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (d0 + j < headdim) row[d0 + j] = v[j];
+  }
+}
+
+// Write a wave's transposed accumulator (DB blocks of 32 headdim rows x 32 sequence columns,
+// lane (c, h) holding sequence position c) to a (seqlen, headdim) tensor.  The values go through
+// a wave-private LDS patch of 32 x (DP + 8) elements so that global stores are 16-byte and
+// row-contiguous.  The caller guarantees the patch is not in use by anyone else.
+template <typename T, int DP>
+__device__ __forceinline__ void store_transposed_acc(const f32x16 (&acc)[DP / 32], float mult,
+                                                     short *patch, short *dst_rows,
+                                                     int64_t stride_seq, int rows_valid,
+                                                     int headdim, bool vec) {
+  constexpr int LD = DP + 8;
+  constexpr int CPR = DP / 8;
+  const int lane = threadIdx.x & 63;
+  const int c = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int db = 0; db < DP / 32; db++) {
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      f32x4 x = {acc[db][4 * g] * mult, acc[db][4 * g + 1] * mult, acc[db][4 * g + 2] * mult,
+                 acc[db][4 * g + 3] * mult};
+      *reinterpret_cast<s16x4 *>(patch + c * LD + 32 * db + 8 * g + 4 * h) = Elem<T>::pack4(x);
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int it = 0; it < (32 * CPR) / 64; it++) {
+    int id = lane + 64 * it;
+    int r = id / CPR, cc = id % CPR;
+    s16x8 v = *reinterpret_cast<const s16x8 *>(patch + r * LD + cc * 8);
+    store_chunk(dst_rows + (int64_t)r * stride_seq, cc * 8, headdim, r < rows_valid, vec, v);
+  }
+}
+
+}  // namespace fa2

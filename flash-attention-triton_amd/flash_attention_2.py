@@ -1,0 +1,380 @@
+"""FlashAttention-2 for AMD MI355X (gfx950): public API and autograd boundary.
+
+Drop-in for ``flash_attention_triton.flash_attention_2`` of the reference
+(src/flash_attention_triton/flash_attention_2.py): same public functions, same
+``torch.autograd.Function`` contract, same assertion and exception types; the device work is
+done by hand-written HIP kernels reached through the C ABI of ``libfa2_gfx950.so``.
+
+Differences from the reference, all deliberate:
+
+* bf16 inputs are computed with bf16 MFMA; the reference down-casts everything to fp16
+  (flash_attention_2.py:316).  fp16 inputs use fp16 MFMA; any other dtype is down-cast to fp16
+  and the output cast back, as in the reference.
+* fp16/bf16 contiguous inputs are used as they are: no cast or copy kernels run.
+* The configuration selector knows one architecture, gfx950.
+* ``deterministic=True`` does not serialise the backward into one program per head
+  (flash_attention_2.py:204-207): dQ is produced by a query-tile-parallel kernel that accumulates
+  in a fixed order without atomics.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _capi
+from ._configurators_v2 import BackwardConfig, KernelsConfigV2, init_to_zero_v2
+
+# Architecture this package is written for, and what torch reports for it.
+_GFX950_ARCH_PREFIX = "gfx950"
+_MIN_CC = (9, 5)
+
+_COMPUTE_DTYPES = {torch.float16: _capi.FA2_DTYPE_F16, torch.bfloat16: _capi.FA2_DTYPE_BF16}
+
+
+# ================================ AUTOGRAD INTEGRATION ================================
+def _strides3(t: torch.Tensor) -> tuple[int, int, int]:
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
+def _stream_handle() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _flash_attention_forward(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    softmax_scale: float | None,
+    block_rows_size: int,
+    block_cols_size: int,
+    min_block_headdim: int,
+    max_headdim: int,
+    seqlen_cache_divisor: int,
+    min_warps: int,
+    max_warps: int,
+    num_stages: int,
+) -> tuple[torch.Tensor, torch.Tensor, float]:
+    """Validate inputs, allocate O and the log-sum-exp, launch the forward kernel.
+
+    Same signature, checks and return value as the reference launcher
+    (flash_attention_2.py:61-144).  The tile arguments are accepted for compatibility; the tile
+    shape comes from the table inside the library.
+    """
+    batch, nheads, seqlen_q, headdim = q.shape
+    _, _, seqlen_k, _ = k.shape
+
+    assert k.shape == (batch, nheads, seqlen_k, headdim)
+    assert v.shape == (batch, nheads, seqlen_k, headdim)
+    assert headdim <= max_headdim, f"Supports head dimensions only up to {max_headdim}"
+    assert q.is_cuda and k.is_cuda and v.is_cuda, "All tensors must reside on CUDA device"
+    assert q.dtype == k.dtype == v.dtype, "All tensors must be the same type"
+    assert q.dtype in _COMPUTE_DTYPES, "Supports only fp16 and bf16"
+    assert q.stride(-1) == k.stride(-1) == v.stride(-1) == 1, "Last dimension must be contiguous"
+
+    output = torch.empty_like(q)
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(headdim)
+
+    # Row length of lse padded to a multiple of max_headdim (reference: flash_attention_2.py:98-99)
+    seqlen_q_rounded = math.ceil(seqlen_q / max_headdim) * max_headdim
+    lse = torch.empty((batch, nheads, seqlen_q_rounded), device=q.device, dtype=torch.float32)
+
+    lib = _capi.load()
+    with torch.cuda.device(q.device):
+        status = lib.fa2_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), lse.data_ptr(),
+            batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded,
+            *_strides3(q), *_strides3(k), *_strides3(v), *_strides3(output),
+            softmax_scale, _COMPUTE_DTYPES[q.dtype], _capi.FA2_CONFIG_AUTO, _stream_handle(),
+        )
+    _capi.check(status, "fa2_fwd")
+    return output, lse, softmax_scale  # softmax_scale could have been updated
+
+
+def _flash_attention_backward(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    output: torch.Tensor,
+    lse: torch.Tensor,
+    dq: torch.Tensor,
+    dk: torch.Tensor,
+    dv: torch.Tensor,
+    d_output: torch.Tensor,
+    softmax_scale: float | None,
+    kernels_config: KernelsConfigV2,
+) -> None:
+    """Fill caller-allocated dq, dk, dv in place (reference: flash_attention_2.py:147-277)."""
+    batch, nheads, seqlen_q, headdim = q.shape
+    _, _, seqlen_k, _ = k.shape
+
+    if not d_output.is_contiguous():
+        d_output = d_output.contiguous()
+
+    max_headdim = kernels_config.max_headdim
+    seqlen_q_rounded = math.ceil(seqlen_q / max_headdim) * max_headdim
+
+    assert headdim <= max_headdim
+    assert lse.shape == (batch, nheads, seqlen_q_rounded)
+    assert (
+        q.is_contiguous()
+        == k.is_contiguous()
+        == v.is_contiguous()
+        == output.is_contiguous()
+        == True  # noqa: E712
+    )
+    assert dq.is_contiguous() == dk.is_contiguous() == dv.is_contiguous() == True  # noqa: E712
+    assert q.dtype in _COMPUTE_DTYPES, "Supports only fp16 and bf16"
+    assert d_output.dtype == q.dtype == output.dtype, "All tensors must be the same type"
+
+    delta = torch.empty_like(lse)
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(headdim)
+    deterministic = 1 if kernels_config.deterministic else 0
+    dtype = _COMPUTE_DTYPES[q.dtype]
+
+    lib = _capi.load()
+    with torch.cuda.device(q.device):
+        stream = _stream_handle()
+        status = lib.fa2_bwd_preprocess(
+            output.data_ptr(), d_output.data_ptr(), delta.data_ptr(),
+            batch, nheads, seqlen_q, headdim, seqlen_q_rounded,
+            *_strides3(output), *_strides3(d_output), dtype, stream,
+        )
+        _capi.check(status, "fa2_bwd_preprocess")
+
+        ws_bytes = lib.fa2_bwd_workspace_bytes(batch, nheads, seqlen_q, seqlen_k, headdim,
+                                               deterministic, _capi.FA2_CONFIG_AUTO)
+        workspace = (torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None)
+        status = lib.fa2_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), d_output.data_ptr(),
+            lse.data_ptr(), delta.data_ptr(),
+            workspace.data_ptr() if workspace is not None else None,
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+            batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded,
+            *_strides3(q), *_strides3(k), *_strides3(v), *_strides3(d_output),
+            *_strides3(dq), *_strides3(dk), *_strides3(dv),
+            softmax_scale, dtype, deterministic, _capi.FA2_CONFIG_AUTO, stream,
+        )
+        _capi.check(status, "fa2_bwd")
+
+
+def _compute_dtype(dtype: torch.dtype) -> torch.dtype:
+    """bf16 stays bf16; everything else is computed in fp16 like the reference."""
+    return torch.bfloat16 if dtype == torch.bfloat16 else torch.float16
+
+
+class FlashAttentionV2Function(torch.autograd.Function):
+    """Autograd function for FlashAttention v2 (reference: flash_attention_2.py:280-384)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, softmax_scale, kernels_config):  # noqa: ANN001, ANN205
+        """Forward pass; saves (q, k, v, o, lse) in the compute dtype for backward."""
+        initial_dtype = q.dtype
+        compute_dtype = _compute_dtype(initial_dtype)
+
+        # No-ops for contiguous fp16/bf16 inputs.
+        q, k, v = [proj.contiguous().to(compute_dtype) for proj in (q, k, v)]
+
+        output, lse, ctx.softmax_scale = _flash_attention_forward(
+            q,
+            k,
+            v,
+            softmax_scale,
+            kernels_config.block_rows_size,
+            kernels_config.block_cols_size,
+            kernels_config.min_block_headdim,
+            kernels_config.max_headdim,
+            kernels_config.seqlen_cache_divisor,
+            kernels_config.min_warps,
+            kernels_config.max_warps,
+            kernels_config.num_stages,
+        )
+
+        ctx.save_for_backward(q, k, v, output, lse)
+        ctx.kernels_config = kernels_config
+
+        return output.contiguous().to(initial_dtype)
+
+    @staticmethod
+    def backward(ctx, d_output):  # noqa: ANN001, ANN205
+        """Gradients for q, k, v; the two non-tensor inputs get None."""
+        q, k, v, output, lse = ctx.saved_tensors
+        kernels_config = ctx.kernels_config
+
+        # Like the reference (flash_attention_2.py:364) the backward is not differentiable.
+        with torch.inference_mode():
+            dq = torch.empty_like(q)
+            dk = torch.empty_like(k)
+            dv = torch.empty_like(v)
+
+            _flash_attention_backward(
+                q,
+                k,
+                v,
+                output,
+                lse,
+                dq,
+                dk,
+                dv,
+                d_output.to(q.dtype),
+                ctx.softmax_scale,
+                kernels_config,
+            )
+
+        return dq, dk, dv, None, None
+
+
+# ============================ gfx950 DEFAULT CONFIGURATIONS ============================
+# Replaces the reference's eight Turing/Ampere x Triton-version constants
+# (flash_attention_2.py:387-565).  The numbers restate the table compiled into the library
+# (csrc/fa2_capi.hip); `_capi.config_table()` returns that table at run time.
+GFX950_BACKWARD_CONFIGS_DETERMINISTIC = [
+    BackwardConfig(
+        {"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": False},
+        num_warps=4,
+        num_stages=2,
+        pre_hook=init_to_zero_v2("DQ"),
+    ),
+]
+GFX950_BACKWARD_CONFIGS_NON_DETERMINISTIC = [
+    BackwardConfig(
+        {"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": True},
+        num_warps=4,
+        num_stages=2,
+        pre_hook=init_to_zero_v2("DQ"),
+    ),
+]
+GFX950_KERNEL_CONFIG_DETERMINISTIC = KernelsConfigV2(
+    block_rows_size=128,
+    block_cols_size=64,
+    min_block_headdim=32,
+    max_headdim=_capi.FA2_MAX_HEADDIM,
+    seqlen_cache_divisor=32,
+    min_warps=4,
+    max_warps=4,
+    num_stages=2,
+    backward_autotune_configs=GFX950_BACKWARD_CONFIGS_DETERMINISTIC,
+)
+GFX950_KERNEL_CONFIG_NON_DETERMINISTIC = KernelsConfigV2(
+    block_rows_size=128,
+    block_cols_size=64,
+    min_block_headdim=32,
+    max_headdim=_capi.FA2_MAX_HEADDIM,
+    seqlen_cache_divisor=32,
+    min_warps=4,
+    max_warps=4,
+    num_stages=2,
+    backward_autotune_configs=GFX950_BACKWARD_CONFIGS_NON_DETERMINISTIC,
+)
+
+_GPU_ARCHITECTURES = {
+    "gfx950": {
+        True: GFX950_KERNEL_CONFIG_DETERMINISTIC,
+        False: GFX950_KERNEL_CONFIG_NON_DETERMINISTIC,
+    },
+}
+
+
+# ========================= INTERNAL HELPERS FOR PUBLIC API =========================
+def _current_arch_name() -> str:
+    props = torch.cuda.get_device_properties(torch.cuda.current_device())
+    return getattr(props, "gcnArchName", "") or ""
+
+
+def _validate_runtime_compatibility(cc: tuple[int, int], arch_name: str | None = None) -> None:
+    """Check that the current device can run the compiled kernels and that they are loadable.
+
+    Plays the role of the reference's _validate_triton_compatibility
+    (flash_attention_2.py:593-614): RuntimeError when the software stack does not fit the GPU.
+    """
+    if arch_name is None:
+        arch_name = _current_arch_name()
+    if not arch_name.startswith(_GFX950_ARCH_PREFIX):
+        raise RuntimeError(
+            f"Device architecture {arch_name!r} (compute capability {cc}) detected; "
+            "libfa2_gfx950.so contains gfx950 (MI355X) code objects only"
+        )
+    _capi.load()  # raises RuntimeError when the library is missing or has the wrong ABI
+
+
+def _select_optimal_gpu_architecture(cc: tuple[int, int], deterministic: bool) -> KernelsConfigV2:
+    """Pick the configuration for the device (reference: flash_attention_2.py:617-642).
+
+    Raises:
+        ValueError: If the compute capability is below what gfx950 reports.
+    """
+    if cc < _MIN_CC:
+        raise ValueError(
+            f"Unsupported GPU compute capability {cc}. Minimum required: {_MIN_CC} (gfx950)"
+        )
+    return _GPU_ARCHITECTURES["gfx950"][bool(deterministic)]
+
+
+# =================================== PUBLIC API ===================================
+def flash_attention_v2(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    softmax_scale: float | None = None,
+    deterministic: bool = False,
+) -> torch.Tensor:
+    """Causal FlashAttention-2 with gfx950 kernels (reference: flash_attention_2.py:646-697).
+
+    Args:
+        q: Query tensor of shape (batch, nheads, seqlen_q, headdim).
+        k: Key tensor of shape (batch, nheads, seqlen_k, headdim).
+        v: Value tensor of shape (batch, nheads, seqlen_k, headdim).
+        softmax_scale: Softmax scaling factor (default: 1/sqrt(headdim)).
+        deterministic: Use the backward whose results are bit-identical from run to run.
+
+    Returns:
+        Attention output tensor, same shape and dtype as q.
+    """
+    cc = torch.cuda.get_device_capability()
+    _validate_runtime_compatibility(cc)
+
+    kernels_config = _select_optimal_gpu_architecture(cc, deterministic)
+
+    return FlashAttentionV2Function.apply(q, k, v, softmax_scale, kernels_config)
+
+
+def flash_attention_v2_custom(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    softmax_scale: float | None,
+    kernels_configs: dict[tuple[int, int], KernelsConfigV2],
+) -> torch.Tensor:
+    """Causal FlashAttention-2 with a caller-supplied configuration per compute capability.
+
+    Same contract as the reference (flash_attention_2.py:700-790): the dictionary is keyed by
+    ``torch.cuda.get_device_capability()`` of the current device ((9, 5) on MI355X); a missing
+    key raises ValueError.
+
+    Example:
+        configs = {(9, 5): KernelsConfigV2(
+            block_rows_size=128, block_cols_size=64, min_block_headdim=32, max_headdim=128,
+            seqlen_cache_divisor=32, min_warps=4, max_warps=4, num_stages=2,
+            backward_autotune_configs=[BackwardConfig(
+                {"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": False},
+                num_warps=4, num_stages=2, pre_hook=init_to_zero_v2("DQ"))])}
+        out = flash_attention_v2_custom(q, k, v, softmax_scale=None, kernels_configs=configs)
+    """
+    cc = torch.cuda.get_device_capability()
+
+    if cc not in kernels_configs:
+        raise ValueError(
+            f"Missing kernel configuration for compute capability {cc}. "
+            "KernelsConfig must be provided for the current GPU architecture"
+        )
+    _validate_runtime_compatibility(cc)
+
+    kernels_config = kernels_configs[cc]
+    if kernels_config.max_headdim > _capi.FA2_MAX_HEADDIM:
+        raise ValueError(
+            f"max_headdim={kernels_config.max_headdim} exceeds what the compiled kernels "
+            f"support ({_capi.FA2_MAX_HEADDIM})"
+        )
+
+    return FlashAttentionV2Function.apply(q, k, v, softmax_scale, kernels_config)

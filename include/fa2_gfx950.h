@@ -1,0 +1,163 @@
+/*
+ * fa2_gfx950.h - C ABI of libfa2_gfx950.so: causal FlashAttention-2 forward and backward
+ * as hand-written HIP kernels for AMD MI355X (gfx950, CDNA4).
+ *
+ * The library replaces the device side of egaoharu-kensei/flash-attention-triton.  Every entry
+ * point cites the reference interface it stands in for (paths relative to the reference
+ * repository root).  Conventions shared by all entry points:
+ *
+ *  - Tensors are (batch, nheads, seqlen, headdim) with element stride 1 on headdim; batch, head
+ *    and sequence strides are passed in ELEMENTS (the reference kernels take the same three
+ *    strides and assume stride 1 on headdim: src/flash_attention_triton/_triton_kernels_v2.py:88-105).
+ *  - Causal masking keeps key column j for query row i when j <= i, anchored at the top-left
+ *    corner also when seqlen_q != seqlen_k (_triton_kernels_v2.py:139-147).
+ *  - The library never allocates, frees or retains device memory: the caller owns every buffer
+ *    (as the reference's Python launchers do, flash_attention_2.py:93-100, 195-196, 365-367).
+ *  - Calls only enqueue work on `stream` (a hipStream_t passed as void*; NULL = the null
+ *    stream) and never synchronise.
+ *  - Every function returns an fa2_status (0 = success).  Nothing throws or aborts; a textual
+ *    description of the last failure on the calling thread is available from
+ *    fa2_last_error_string().
+ *  - lse and delta are fp32 arrays of shape (batch, nheads, seqlen_q_rounded) where
+ *    seqlen_q_rounded >= seqlen_q is chosen by the caller (the reference pads the row length to
+ *    a multiple of max_headdim, flash_attention_2.py:98-99).  Rows [seqlen_q, seqlen_q_rounded)
+ *    are written with zeros.
+ */
+#ifndef FA2_GFX950_H
+#define FA2_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FA2_ABI_VERSION 1
+
+/* Largest head dimension the kernels accept (the table's `max_headdim`). */
+#define FA2_MAX_HEADDIM 128
+
+typedef enum fa2_status {
+  FA2_OK = 0,
+  FA2_ERR_NULL_POINTER = 1,     /* a required device pointer is NULL */
+  FA2_ERR_BAD_SHAPE = 2,        /* non-positive size, or seqlen_q_rounded < seqlen_q */
+  FA2_ERR_BAD_DTYPE = 3,        /* dtype is neither FA2_DTYPE_F16 nor FA2_DTYPE_BF16 */
+  FA2_ERR_HEADDIM = 4,          /* headdim > FA2_MAX_HEADDIM */
+  FA2_ERR_BAD_STRIDE = 5,       /* negative stride */
+  FA2_ERR_BAD_CONFIG = 6,       /* config id outside the table, or not valid for this problem */
+  FA2_ERR_WORKSPACE = 7,        /* a workspace is required but NULL */
+  FA2_ERR_LAUNCH = 8,           /* hipLaunchKernel reported an error */
+  FA2_ERR_TOO_LARGE = 9         /* a size or offset exceeds what the kernels index */
+} fa2_status;
+
+typedef enum fa2_dtype {
+  FA2_DTYPE_F16 = 0, /* IEEE half: the reference's only compute type (flash_attention_2.py:90) */
+  FA2_DTYPE_BF16 = 1 /* bfloat16 on bf16 MFMA; the reference down-casts bf16 to fp16 instead */
+} fa2_dtype;
+
+/* Ask the table to choose (pass as config_id). */
+#define FA2_CONFIG_AUTO (-1)
+
+/*
+ * One row of the gfx950 tile/wave table.  Replaces the reference's per-architecture
+ * KernelsConfigV2 constants and their selector (flash_attention_2.py:387-642).
+ */
+typedef struct fa2_config_info {
+  int id;
+  int headdim_padded; /* head dimension the kernels are instantiated for (>= headdim) */
+  int fwd_block_q;    /* query rows per workgroup, forward */
+  int fwd_block_kv;   /* key rows per inner step, forward */
+  int fwd_waves;      /* wavefronts (64 lanes) per workgroup, forward */
+  int bwd_block_q;    /* query rows per inner step, dK/dV kernel */
+  int bwd_block_kv;   /* key rows per workgroup, dK/dV kernel */
+  int bwd_waves;
+  int dq_block_q;     /* query rows per workgroup, dQ kernel (deterministic mode) */
+  int dq_block_kv;
+  int dq_waves;
+} fa2_config_info;
+
+/* ABI version of the loaded library; equals FA2_ABI_VERSION of the header it was built from. */
+int fa2_abi_version(void);
+
+/* Description of the most recent failure on the calling thread ("" if none). */
+const char *fa2_last_error_string(void);
+
+/* Static name of a status code. */
+const char *fa2_status_string(int status);
+
+/* Number of rows in the gfx950 table. */
+int fa2_config_count(void);
+
+/* Copy table row `config_id` to *out. */
+int fa2_config_get(int config_id, fa2_config_info *out);
+
+/*
+ * Table lookup: replaces _select_optimal_gpu_architecture (flash_attention_2.py:617-642).
+ * Returns the row id (>= 0) chosen for the problem, or a negative fa2_status on error.
+ */
+int fa2_pick_config(int dtype, int headdim, int seqlen_q, int seqlen_k, int deterministic);
+
+/*
+ * Forward: O = softmax(scale * Q K^T + causal mask) V and the row log-sum-exp.
+ * Replaces _flash_attention_forward + _forward_kernel
+ * (flash_attention_2.py:61-144, _triton_kernels_v2.py:11-189).
+ * q, o: (batch, nheads, seqlen_q, headdim); k, v: (batch, nheads, seqlen_k, headdim);
+ * lse: fp32 (batch, nheads, seqlen_q_rounded), natural-log units.
+ */
+int fa2_fwd(const void *q, const void *k, const void *v, void *o, float *lse,
+            int batch, int nheads, int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded,
+            int64_t q_stride_batch, int64_t q_stride_head, int64_t q_stride_seq,
+            int64_t k_stride_batch, int64_t k_stride_head, int64_t k_stride_seq,
+            int64_t v_stride_batch, int64_t v_stride_head, int64_t v_stride_seq,
+            int64_t o_stride_batch, int64_t o_stride_head, int64_t o_stride_seq,
+            float softmax_scale, int dtype, int config_id, void *stream);
+
+/*
+ * Backward preprocess: delta[b,h,i] = sum_d O[b,h,i,d] * dO[b,h,i,d] in fp32.
+ * Replaces _backward_preprocess_do_o_dot (_triton_kernels_v2.py:532-608; launched at
+ * flash_attention_2.py:218-234).
+ */
+int fa2_bwd_preprocess(const void *o, const void *d_o, float *delta,
+                       int batch, int nheads, int seqlen_q, int headdim, int seqlen_q_rounded,
+                       int64_t o_stride_batch, int64_t o_stride_head, int64_t o_stride_seq,
+                       int64_t do_stride_batch, int64_t do_stride_head, int64_t do_stride_seq,
+                       int dtype, void *stream);
+
+/*
+ * Bytes of fp32 workspace fa2_bwd needs for dQ accumulation (0 when the chosen mode writes dQ
+ * directly).  Stands in for the reference's dq_accum allocation (flash_attention_2.py:196).
+ */
+size_t fa2_bwd_workspace_bytes(int batch, int nheads, int seqlen_q, int seqlen_k, int headdim,
+                               int deterministic, int config_id);
+
+/*
+ * Backward main: fills dq, dk, dv (same dtype as q) in place.
+ * Replaces _flash_attention_backward's main launch, the dQ zero-fill pre-hook and the final
+ * dq.copy_(dq_accum) (flash_attention_2.py:235-277, _configurators_v2.py:81-93,
+ * _triton_kernels_v2.py:192-529).
+ *   deterministic != 0: dQ is accumulated in a fixed order without atomics; results are
+ *                       bit-identical from run to run.
+ *   deterministic == 0: dQ may be accumulated with fp32 atomic adds into `workspace`
+ *                       (sequence-parallel mode); low-order bits can differ between runs.
+ * `workspace` must hold fa2_bwd_workspace_bytes(...) bytes (may be NULL when that is 0); the
+ * library clears what it needs.
+ */
+int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o,
+            const float *lse, const float *delta, void *workspace,
+            void *dq, void *dk, void *dv,
+            int batch, int nheads, int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded,
+            int64_t q_stride_batch, int64_t q_stride_head, int64_t q_stride_seq,
+            int64_t k_stride_batch, int64_t k_stride_head, int64_t k_stride_seq,
+            int64_t v_stride_batch, int64_t v_stride_head, int64_t v_stride_seq,
+            int64_t do_stride_batch, int64_t do_stride_head, int64_t do_stride_seq,
+            int64_t dq_stride_batch, int64_t dq_stride_head, int64_t dq_stride_seq,
+            int64_t dk_stride_batch, int64_t dk_stride_head, int64_t dk_stride_seq,
+            int64_t dv_stride_batch, int64_t dv_stride_head, int64_t dv_stride_seq,
+            float softmax_scale, int dtype, int deterministic, int config_id, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FA2_GFX950_H */
