@@ -1,0 +1,206 @@
+"""CPU-only tests: the oracle against the golden fixtures, the C-ABI library's exports and
+argument validation (no kernel is launched), and the Python boundary's contract."""
+
+from __future__ import annotations
+
+import ctypes
+import dataclasses
+import pathlib
+import re
+
+import pytest
+import torch
+
+from oracle import naive_attention as oracle
+from tests import golden_io
+
+ROOT = pathlib.Path(__file__).resolve().parent.parent
+
+
+# ------------------------------------------------------------------ oracle vs golden fixtures
+@pytest.mark.parametrize("name", golden_io.NAMES)
+def test_oracle_reproduces_golden_fixture(name):
+    g = golden_io.load(name)
+    o, dq, dk, dv = oracle.naive_backward(g["q"], g["k"], g["v"], g["d_o"], g["scale"], torch.float32)
+    lse = oracle.naive_lse(g["q"], g["k"], g["scale"])
+    for got, key in ((o, "o"), (dq, "dq"), (dk, "dk"), (dv, "dv"), (lse, "lse")):
+        torch.testing.assert_close(got, g[key], atol=2e-5, rtol=2e-5)
+
+
+# ------------------------------------------------------------------ C ABI: exports and errors
+def _declared_functions() -> list[str]:
+    text = (ROOT / "include" / "fa2_gfx950.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b(fa2_[a-z0-9_]+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol(capi):
+    lib = capi.load()
+    names = sorted(set(_declared_functions()))
+    assert names, "no declarations found in include/fa2_gfx950.h"
+    for name in names:
+        assert hasattr(lib, name), f"libfa2_gfx950.so does not export {name}"
+    assert sorted(capi.SIGNATURES) == names, "ctypes binding and header disagree on the entry points"
+
+
+def test_abi_version_and_table(capi):
+    lib = capi.load()
+    assert lib.fa2_abi_version() == capi.ABI_VERSION
+    rows = capi.config_table()
+    assert [r["headdim_padded"] for r in rows] == sorted(r["headdim_padded"] for r in rows)
+    assert rows[-1]["headdim_padded"] == capi.FA2_MAX_HEADDIM
+    for r in rows:
+        assert r["fwd_block_q"] == 32 * r["fwd_waves"]
+        assert r["bwd_block_kv"] == 32 * r["bwd_waves"]
+        assert r["dq_block_q"] == 32 * r["dq_waves"]
+    for d, want in ((1, 32), (32, 32), (33, 64), (48, 64), (64, 64), (96, 96), (100, 128), (128, 128)):
+        idx = lib.fa2_pick_config(capi.FA2_DTYPE_BF16, d, 512, 512, 0)
+        assert idx >= 0 and rows[idx]["headdim_padded"] == want
+    assert lib.fa2_pick_config(capi.FA2_DTYPE_BF16, 129, 512, 512, 0) == -4  # FA2_ERR_HEADDIM
+    assert lib.fa2_pick_config(7, 64, 512, 512, 0) == -3  # FA2_ERR_BAD_DTYPE
+    info = capi.ConfigInfo()
+    assert lib.fa2_config_get(99, ctypes.byref(info)) == 6  # FA2_ERR_BAD_CONFIG
+    assert lib.fa2_config_get(0, None) == 1  # FA2_ERR_NULL_POINTER
+
+
+def _fwd_args(capi, **over):
+    a = dict(q=16, k=16, v=16, o=16, lse=16, batch=1, nheads=1, seqlen_q=8, seqlen_k=8, headdim=64,
+             seqlen_q_rounded=128, scale=0.125, dtype=capi.FA2_DTYPE_F16, config=capi.FA2_CONFIG_AUTO)
+    a.update(over)
+    strides = [a["seqlen_q"] * a["headdim"], a["seqlen_q"] * a["headdim"], a["headdim"]] * 4
+    if "strides" in over:
+        strides = over["strides"]
+    return [a["q"], a["k"], a["v"], a["o"], a["lse"], a["batch"], a["nheads"], a["seqlen_q"], a["seqlen_k"],
+            a["headdim"], a["seqlen_q_rounded"], *strides, a["scale"], a["dtype"], a["config"], None]
+
+
+@pytest.mark.parametrize("over,status", [
+    (dict(q=None), "FA2_ERR_NULL_POINTER"),
+    (dict(lse=None), "FA2_ERR_NULL_POINTER"),
+    (dict(batch=0), "FA2_ERR_BAD_SHAPE"),
+    (dict(seqlen_k=-3), "FA2_ERR_BAD_SHAPE"),
+    (dict(seqlen_q=300, seqlen_q_rounded=256), "FA2_ERR_BAD_SHAPE"),
+    (dict(headdim=136), "FA2_ERR_HEADDIM"),
+    (dict(dtype=5), "FA2_ERR_BAD_DTYPE"),
+    (dict(config=17), "FA2_ERR_BAD_CONFIG"),
+    (dict(config=0, headdim=64), "FA2_ERR_BAD_CONFIG"),  # row 0 is built for headdim <= 32
+    (dict(scale=float("nan")), "FA2_ERR_BAD_SHAPE"),
+    (dict(strides=[-1] * 12), "FA2_ERR_BAD_STRIDE"),
+])
+def test_forward_rejects_bad_arguments_before_launching(capi, over, status):
+    """Every error returns a status and a message; nothing is launched, thrown or aborted."""
+    lib = capi.load()
+    rc = lib.fa2_fwd(*_fwd_args(capi, **over))
+    assert rc != 0
+    assert lib.fa2_status_string(rc).decode() == status
+    assert lib.fa2_last_error_string().decode() != ""
+    with pytest.raises(RuntimeError, match=status):
+        capi.check(rc, "fa2_fwd")
+
+
+def test_backward_entry_points_reject_bad_arguments(capi):
+    lib = capi.load()
+    st = [512, 512, 64]
+    rc = lib.fa2_bwd_preprocess(None, 16, 16, 1, 1, 8, 64, 128, *st, *st, capi.FA2_DTYPE_F16, None)
+    assert lib.fa2_status_string(rc).decode() == "FA2_ERR_NULL_POINTER"
+    rc = lib.fa2_bwd_preprocess(16, 16, 16, 1, 1, 8, 300, 128, *st, *st, capi.FA2_DTYPE_F16, None)
+    assert lib.fa2_status_string(rc).decode() == "FA2_ERR_HEADDIM"
+    rc = lib.fa2_bwd(16, 16, 16, 16, 16, None, None, 16, 16, 16, 1, 1, 8, 8, 64, 128, *(st * 7),
+                     0.125, capi.FA2_DTYPE_F16, 1, capi.FA2_CONFIG_AUTO, None)
+    assert lib.fa2_status_string(rc).decode() == "FA2_ERR_NULL_POINTER"
+    assert "delta" in lib.fa2_last_error_string().decode()
+    rc = lib.fa2_bwd(16, 16, 16, 16, 16, 16, None, 16, 16, 16, 1, 1, 0, 8, 64, 128, *(st * 7),
+                     0.125, capi.FA2_DTYPE_F16, 1, capi.FA2_CONFIG_AUTO, None)
+    assert lib.fa2_status_string(rc).decode() == "FA2_ERR_BAD_SHAPE"
+    assert lib.fa2_bwd_workspace_bytes(2, 4, 512, 512, 64, 1, capi.FA2_CONFIG_AUTO) == 0
+
+
+def test_missing_library_fails_loudly(capi, monkeypatch, tmp_path):
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIBRARY_PATH", tmp_path / "libfa2_gfx950.so")
+    with pytest.raises(RuntimeError, match="not built"):
+        capi.load()
+
+
+# ------------------------------------------------------------------ Python boundary contract
+def test_public_names_match_reference(fa):
+    """Reference: src/flash_attention_triton/__init__.py:13."""
+    for name in ("KernelsConfigV2", "flash_attention_v2", "flash_attention_v2_custom", "init_to_zero_v2"):
+        assert name in fa.__all__ and hasattr(fa, name)
+
+
+def test_kernels_config_is_a_frozen_record_with_reference_fields(fa):
+    fields = [f.name for f in dataclasses.fields(fa.KernelsConfigV2)]
+    assert fields == ["block_rows_size", "block_cols_size", "min_block_headdim", "max_headdim",
+                      "seqlen_cache_divisor", "min_warps", "max_warps", "num_stages",
+                      "backward_autotune_configs"]
+    cfg = fa.KernelsConfigV2(128, 64, 32, 128, 32, 4, 4, 2, [
+        fa.BackwardConfig({"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": False},
+                          num_warps=4, num_stages=2, pre_hook=fa.init_to_zero_v2("DQ"))])
+    with pytest.raises(dataclasses.FrozenInstanceError):
+        cfg.block_rows_size = 64
+    assert cfg.deterministic is True
+    serial = cfg._serialize_bwd(cfg.backward_autotune_configs)
+    assert serial == (((64, 128, False), 4, 2, "init_to_zero_v2.<locals>.<lambda>"),)
+    hash(serial)
+    par = dataclasses.replace(cfg, backward_autotune_configs=[
+        fa.BackwardConfig({"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": True})])
+    assert par.deterministic is False
+
+
+def test_init_to_zero_hook_zeroes_named_tensor(fa):
+    hook = fa.init_to_zero_v2("DQ")
+    t = torch.ones(4)
+    assert hook({"DQ": t, "DK": torch.ones(2)}) is t
+    assert torch.count_nonzero(t) == 0
+
+
+def test_selector_and_validation(fa2_module, monkeypatch):
+    sel = fa2_module._select_optimal_gpu_architecture
+    assert sel((9, 5), True) is fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC
+    assert sel((9, 5), False) is fa2_module.GFX950_KERNEL_CONFIG_NON_DETERMINISTIC
+    assert sel((9, 5), True).deterministic and not sel((9, 5), False).deterministic
+    with pytest.raises(ValueError, match="Unsupported GPU compute capability"):
+        sel((9, 4), False)
+    with pytest.raises(RuntimeError, match="gfx950"):
+        fa2_module._validate_runtime_compatibility((9, 4), "gfx942:sramecc+:xnack-")
+    fa2_module._validate_runtime_compatibility((9, 5), "gfx950:sramecc+:xnack-")
+
+    # flash_attention_v2_custom: a missing key for the current device is a ValueError
+    monkeypatch.setattr(torch.cuda, "get_device_capability", lambda *a, **k: (9, 5))
+    q = torch.zeros(1, 1, 4, 8)
+    with pytest.raises(ValueError, match="Missing kernel configuration"):
+        fa2_module.flash_attention_v2_custom(q, q, q, None, {(8, 0): sel((9, 5), True)})
+
+
+def test_launcher_assertions_mirror_reference(fa2_module):
+    """Same AssertionErrors as flash_attention_2.py:85-90, raised before any FFI call."""
+    cfg = fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC
+    tail = (cfg.block_rows_size, cfg.block_cols_size, cfg.min_block_headdim, cfg.max_headdim,
+            cfg.seqlen_cache_divisor, cfg.min_warps, cfg.max_warps, cfg.num_stages)
+    fwd = fa2_module._flash_attention_forward
+    q = torch.zeros(1, 2, 8, 16, dtype=torch.float16)
+    with pytest.raises(AssertionError):
+        fwd(q, torch.zeros(1, 2, 8, 32, dtype=torch.float16), q, None, *tail)  # k shape
+    with pytest.raises(AssertionError):
+        fwd(q, q, torch.zeros(1, 3, 8, 16, dtype=torch.float16), None, *tail)  # v shape
+    big = torch.zeros(1, 1, 4, 256, dtype=torch.float16)
+    with pytest.raises(AssertionError, match="Supports head dimensions only up to 128"):
+        fwd(big, big, big, None, *tail)
+    with pytest.raises(AssertionError, match="must reside on CUDA device"):
+        fwd(q, q, q, None, *tail)
+
+
+def test_workload_table_matches_baseline(workloads):
+    w = workloads.WORKLOADS
+    assert w["C1"].shape == (2, 4, 512, 64) and w["C1"].dtype == torch.float16
+    assert w["C2"].shape == (4, 16, 2048, 64) and w["C2"].dtype == torch.bfloat16 and w["C2"].both_modes
+    assert w["C3"].shape == (2, 32, 4096, 128) and w["C3"].dtype == torch.bfloat16
+    assert w["C4"].shape == (1, 16, 16384, 128) and w["C4"].both_modes
+    assert w["C5"].shape == (8, 12, 3000, 64) and w["C5"].qk_std == 3.0
+    assert w["C3"].fwd_flops == pytest.approx(274.88e9, rel=1e-3)
+    assert w["C3"].fwd_bytes == pytest.approx(269.5e6, rel=1e-3)
+    q, k, v, g = workloads.make_inputs(w["C1"])
+    q2, *_ = workloads.make_inputs(w["C1"], heads=3)
+    assert q.dtype == torch.float16 and q.shape == (2, 4, 512, 64)
+    torch.testing.assert_close(q2[:, 0], q.reshape(8, 512, 64)[:3], atol=0, rtol=0)

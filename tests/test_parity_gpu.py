@@ -1,0 +1,319 @@
+"""GPU parity tests: the HIP kernels, called through the public API and the C ABI, against the
+oracle (naive fp32 causal attention) on the same seeded inputs.
+
+Tolerance for O, dQ, dK, dV: ``allclose(atol=2e-2, rtol=1e-2)`` against the fp32 naive result
+computed from the same half-precision inputs (the fallback bar of the task statement; the
+"2x the Triton kernel's error" form cannot be evaluated because the reference kernels cannot
+run beside these).  Deterministic mode: bit-identical across reruns.
+"""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import naive_attention as oracle
+from tests import golden_io
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 2e-2, 1e-2
+
+
+def _assert_close(name, got, want, atol=ATOL, rtol=RTOL):
+    got = got.detach().float().cpu()
+    want = want.detach().float().cpu()
+    assert got.shape == want.shape, f"{name}: shape {tuple(got.shape)} != {tuple(want.shape)}"
+    assert not torch.isnan(got).any(), f"{name} contains NaN"
+    err = (got - want).abs()
+    bad = err > atol + rtol * want.abs()
+    assert not bad.any(), (f"{name}: {int(bad.sum())} of {bad.numel()} elements outside atol={atol} rtol={rtol}; "
+                           f"max abs err {err.max().item():.3e} (reference max {want.abs().max().item():.3e})")
+
+
+def _seeded(shape_q, shape_k, dtype, qk_std=1.0, seed=42):
+    gen = torch.Generator().manual_seed(seed)
+    q = (torch.randn(shape_q, generator=gen) * qk_std).to(dtype)
+    k = (torch.randn(shape_k, generator=gen) * qk_std).to(dtype)
+    v = torch.randn(shape_k, generator=gen).to(dtype)
+    d_o = torch.randn(shape_q, generator=gen).to(dtype)
+    return q, k, v, d_o
+
+
+def _run(fa, q, k, v, d_o, scale, deterministic):
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = fa.flash_attention_v2(qg, kg, vg, scale, deterministic)
+    out.backward(d_o.cuda())
+    torch.cuda.synchronize()
+    return out.detach(), qg.grad, kg.grad, vg.grad
+
+
+def _gpu_fp32_oracle(q, k, v, d_o, scale):
+    """The oracle's own code on the GPU in fp32 (full-precision matmul), one head at a time."""
+    torch.backends.cuda.matmul.allow_tf32 = False
+    torch.set_float32_matmul_precision("highest")
+    return oracle.sliced_forward_backward(q.cuda(), k.cuda(), v.cuda(), d_o.cuda(), scale, torch.float32)
+
+
+# ------------------------------------------------------------------------- small shapes vs CPU oracle
+SMALL_CASES = [
+    # (B, H, Nq, Nk, D, dtype, qk_std)
+    (1, 1, 128, 128, 128, torch.bfloat16, 1.0),
+    (2, 4, 512, 512, 64, torch.float16, 1.0),
+    (1, 2, 75, 75, 64, torch.float16, 1.0),       # shorter than one tile
+    (1, 2, 300, 300, 128, torch.bfloat16, 1.0),   # ragged tail
+    (2, 3, 333, 200, 48, torch.float16, 1.0),     # more queries than keys, padded head dim
+    (2, 3, 200, 333, 96, torch.bfloat16, 1.0),    # more keys than queries
+    (1, 2, 130, 130, 32, torch.float16, 1.0),
+    (1, 2, 100, 100, 40, torch.bfloat16, 1.0),    # head dim multiple of 8 but not of 16
+    (1, 2, 100, 100, 50, torch.float16, 1.0),     # head dim not a multiple of 8: scalar access path
+    (1, 1, 1, 1, 64, torch.float16, 1.0),         # single token
+    (1, 2, 1, 77, 64, torch.bfloat16, 1.0),
+    (1, 2, 77, 1, 64, torch.bfloat16, 1.0),
+    (1, 4, 640, 640, 64, torch.float16, 3.0),     # peaky softmax
+    (1, 2, 257, 257, 128, torch.float16, 1.0),
+]
+
+
+@pytest.mark.parametrize("deterministic", [True, False], ids=["det", "seqpar"])
+@pytest.mark.parametrize("case", SMALL_CASES, ids=lambda c: f"B{c[0]}H{c[1]}Nq{c[2]}Nk{c[3]}D{c[4]}{str(c[5])[6:]}s{c[6]:g}")
+def test_small_shapes_match_cpu_oracle(fa, case, deterministic):
+    b, h, nq, nk, d, dtype, std = case
+    q, k, v, d_o = _seeded((b, h, nq, d), (b, h, nk, d), dtype, std)
+    scale = 1.0 / math.sqrt(d)
+    want = oracle.naive_backward(q, k, v, d_o, scale, torch.float32)
+    got = _run(fa, q, k, v, d_o, scale, deterministic)
+    for name, g, w in zip(("o", "dq", "dk", "dv"), got, want):
+        assert g.dtype == dtype
+        _assert_close(name, g, w)
+
+
+@pytest.mark.parametrize("name", golden_io.NAMES)
+def test_golden_fixtures(fa, fa2_module, name):
+    g = golden_io.load(name)
+    out, dq, dk, dv = _run(fa, g["q"], g["k"], g["v"], g["d_o"], g["scale"], True)
+    for key, got in (("o", out), ("dq", dq), ("dk", dk), ("dv", dv)):
+        _assert_close(key, got, g[key])
+
+
+# ------------------------------------------------------------------------- lse and delta through the launchers / C ABI
+@pytest.mark.parametrize("name", golden_io.NAMES)
+def test_lse_and_delta_match_oracle(fa2_module, capi, name):
+    g = golden_io.load(name)
+    cfg = fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC
+    q, k, v, d_o = (g[x].cuda() for x in ("q", "k", "v", "d_o"))
+    out, lse, scale = fa2_module._flash_attention_forward(
+        q, k, v, g["scale"], cfg.block_rows_size, cfg.block_cols_size, cfg.min_block_headdim,
+        cfg.max_headdim, cfg.seqlen_cache_divisor, cfg.min_warps, cfg.max_warps, cfg.num_stages)
+    b, h, nq, d = q.shape
+    n_r = math.ceil(nq / cfg.max_headdim) * cfg.max_headdim
+    assert lse.shape == (b, h, n_r) and lse.dtype == torch.float32
+    _assert_close("lse", lse[..., :nq], g["lse"], atol=2e-3, rtol=1e-3)
+    assert torch.count_nonzero(lse[..., nq:]) == 0, "padded lse rows must be written as zero"
+
+    delta = torch.full_like(lse, float("nan"))
+    lib = capi.load()
+    s3 = fa2_module._strides3
+    rc = lib.fa2_bwd_preprocess(out.data_ptr(), d_o.data_ptr(), delta.data_ptr(), b, h, nq, d, n_r,
+                                *s3(out), *s3(d_o), fa2_module._COMPUTE_DTYPES[q.dtype],
+                                torch.cuda.current_stream().cuda_stream)
+    capi.check(rc, "fa2_bwd_preprocess")
+    torch.cuda.synchronize()
+    want = oracle.naive_delta(out.cpu(), d_o.cpu())  # from the half-precision O the kernel saved
+    _assert_close("delta", delta[..., :nq], want, atol=1e-3, rtol=1e-4)
+    assert torch.count_nonzero(delta[..., nq:]) == 0
+    _assert_close("delta vs exact", delta[..., :nq], g["delta"], atol=3e-2, rtol=1e-2)
+
+
+# ------------------------------------------------------------------------- BASELINE configurations at full size
+def _workload_case(workloads, name):
+    w = workloads.WORKLOADS[name]
+    q, k, v, d_o = workloads.make_inputs(w, "cpu")
+    return w, q, k, v, d_o
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
+def test_baseline_configs_match_oracle(fa, workloads, name):
+    """Full-size parity.  C1 against the CPU oracle on every head; the larger ones against the CPU
+    oracle on two heads and against the same oracle code run in fp32 on the GPU on every head."""
+    w, q, k, v, d_o = _workload_case(workloads, name)
+    modes = (True, False) if w.both_modes else (False,)
+    cpu_heads = w.batch * w.nheads if name == "C1" else 2
+    if name == "C4":
+        cpu_heads = 1
+    flat = lambda t: t.reshape(w.batch * w.nheads, w.seqlen, w.headdim)  # noqa: E731
+    cpu_want = oracle.sliced_forward_backward(q, k, v, d_o, w.softmax_scale, torch.float32, heads=cpu_heads)
+    gpu_want = None if name == "C1" else _gpu_fp32_oracle(q, k, v, d_o, w.softmax_scale)
+    for deterministic in modes:
+        got = _run(fa, q, k, v, d_o, w.softmax_scale, deterministic)
+        for key, g, cw in zip(("o", "dq", "dk", "dv"), got, cpu_want):
+            _assert_close(f"{name} {key} (cpu oracle, det={deterministic})", flat(g)[:cpu_heads], cw)
+        if gpu_want is not None:
+            for key, g, gw in zip(("o", "dq", "dk", "dv"), got, gpu_want):
+                _assert_close(f"{name} {key} (fp32 oracle on gpu, det={deterministic})", g, gw)
+        # size-independent properties
+        o, dq, dk, dv = (t.float() for t in got)
+        torch.testing.assert_close(o[:, :, 0], v.cuda().float()[:, :, 0], atol=1e-6, rtol=0)  # row 0 == v[0]
+        lhs = (q.cuda().float() * dq).sum((-1, -2))
+        rhs = (k.cuda().float() * dk).sum((-1, -2))
+        scale_ref = (q.cuda().float() * dq).abs().sum((-1, -2))
+        assert ((lhs - rhs).abs() <= 2e-2 * scale_ref + 1e-2).all(), "sum(q*dq) != sum(k*dk)"
+        torch.testing.assert_close(dv.sum(-2), d_o.cuda().float().sum(-2), atol=0.02 * math.sqrt(w.seqlen), rtol=2e-2)
+
+
+def test_constant_values_give_constant_output(fa, workloads):
+    """V == 1 makes O == 1 exactly representable: checks the normalisation at full C3 size."""
+    w, q, k, v, d_o = _workload_case(workloads, "C3")
+    out = fa.flash_attention_v2(q.cuda(), k.cuda(), torch.ones_like(v).cuda())
+    torch.testing.assert_close(out.float(), torch.ones_like(out, dtype=torch.float32), atol=8e-3, rtol=0)
+
+
+# ------------------------------------------------------------------------- determinism
+@pytest.mark.parametrize("name,reruns", [("C1", 100), ("C2", 10), ("C4", 3), ("C5", 5)])
+def test_determinism(fa, workloads, name, reruns):
+    """deterministic=True is bit-identical from run to run (reference: tests/test_flash_attention_2.py:321-342)."""
+    w, q, k, v, d_o = _workload_case(workloads, name)
+    ref = _run(fa, q, k, v, d_o, w.softmax_scale, True)
+    for i in range(reruns):
+        got = _run(fa, q, k, v, d_o, w.softmax_scale, True)
+        for key, a, b in zip(("output", "dq", "dk", "dv"), got, ref):
+            assert torch.equal(a, b), f"Non-determinism detected in deterministic mode at rerun {i} for {key}"
+
+
+def test_non_determinism(fa, workloads):
+    """deterministic=False may differ between reruns; like the reference's test
+    (tests/test_flash_attention_2.py:345-385) this only reports when it does not."""
+    w, q, k, v, d_o = _workload_case(workloads, "C2")
+    ref = _run(fa, q, k, v, d_o, w.softmax_scale, False)
+    differs = False
+    for _ in range(5):
+        got = _run(fa, q, k, v, d_o, w.softmax_scale, False)
+        differs |= any(not torch.equal(a, b) for a, b in zip(got, ref))
+    if not differs:
+        pytest.skip("non-deterministic mode produced identical bits in 5 reruns (allowed)")
+
+
+# ------------------------------------------------------------------------- the reference's own test matrix
+REFERENCE_SHAPES = [(8, 12, 512, 32), (16, 16, 1024, 48), (32, 20, 1024, 64), (32, 20, 1024, 96), (64, 32, 2048, 128)]
+REFERENCE_IDS = ["small", "medium", "medium+", "large", "large+"]
+
+
+def _reference_inputs(shape):
+    """fp32 inputs on the GPU with requires_grad, as tests/test_flash_attention_2.py:55-72 builds them."""
+    torch.manual_seed(42)
+    q, k, v = (torch.randn(shape, dtype=torch.float32, device="cuda", requires_grad=True) for _ in range(3))
+    return q, k, v, 1.0 / math.sqrt(shape[-1])
+
+
+@pytest.mark.parametrize("shape", REFERENCE_SHAPES, ids=REFERENCE_IDS)
+def test_reference_matrix_forward(fa, shape):
+    """Output shape, dtype, NaN-freeness and agreement with vanilla attention and torch SDPA on
+    fp32 inputs with the reference's own tolerance (tests/test_flash_attention_2.py:236-318)."""
+    q, k, v, scale = _reference_inputs(shape)
+    out = fa.flash_attention_v2(q, k, v, scale)
+    assert out.shape == q.shape and out.dtype == torch.float32
+    assert not torch.isnan(out).any()
+    with torch.no_grad():
+        sdpa = F.scaled_dot_product_attention(q, k, v, is_causal=True, scale=scale)
+        assert torch.allclose(out, sdpa, atol=1e-2, rtol=1e-3), "output doesn't match torch SDPA"
+        heads = min(4, shape[0] * shape[1])
+        flat = lambda t: t.reshape(-1, 1, shape[2], shape[3])[:heads]  # noqa: E731
+        vanilla = oracle.naive_causal_attention(flat(q), flat(k), flat(v), scale)
+        assert torch.allclose(flat(out), vanilla, atol=1e-2, rtol=1e-3), "output doesn't match vanilla attention"
+
+
+@pytest.mark.parametrize("shape", REFERENCE_SHAPES[:4], ids=REFERENCE_IDS[:4])
+def test_reference_matrix_gradients(fa, shape):
+    """Gradients exist in the input dtype, hold no NaN, and match autograd of vanilla attention
+    (the reference only checks for NaN: tests/test_flash_attention_2.py:256-271)."""
+    q, k, v, scale = _reference_inputs(shape)
+    d_o = torch.randn_like(q)
+    fa.flash_attention_v2(q, k, v, scale).backward(d_o)
+    for t in (q, k, v):
+        assert t.grad is not None and t.grad.dtype == torch.float32 and not torch.isnan(t.grad).any()
+    heads = min(4, shape[0] * shape[1])
+    flat = lambda t: t.detach().reshape(-1, 1, shape[2], shape[3])[:heads]  # noqa: E731
+    _, dq, dk, dv = oracle.naive_backward(flat(q), flat(k), flat(v), flat(d_o), scale, torch.float32)
+    _assert_close("dq", flat(q.grad), dq)
+    _assert_close("dk", flat(k.grad), dk)
+    _assert_close("dv", flat(v.grad), dv)
+
+
+def test_flash_attention_v2_custom_equals_default(fa, fa2_module):
+    """A custom configuration equal to the default gives bit-identical O, dQ, dK, dV
+    (tests/test_flash_attention_2.py:388-411)."""
+    q, k, v, d_o = _seeded((4, 6, 512, 64), (4, 6, 512, 64), torch.float16)
+    cc = torch.cuda.get_device_capability()
+    configs = {cc: fa.KernelsConfigV2(
+        block_rows_size=128, block_cols_size=64, min_block_headdim=32, max_headdim=128,
+        seqlen_cache_divisor=32, min_warps=4, max_warps=4, num_stages=2,
+        backward_autotune_configs=[fa.BackwardConfig(
+            {"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": False},
+            num_warps=4, num_stages=2, pre_hook=fa.init_to_zero_v2("DQ"))])}
+    ref = _run(fa, q, k, v, d_o, None, True)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = fa.flash_attention_v2_custom(qg, kg, vg, None, configs)
+    out.backward(d_o.cuda())
+    for key, a, b in zip(("output", "dq", "dk", "dv"), (out.detach(), qg.grad, kg.grad, vg.grad), ref):
+        assert torch.equal(a, b), f"custom configuration differs from default for {key}"
+    with pytest.raises(ValueError, match="Missing kernel configuration"):
+        fa.flash_attention_v2_custom(qg, kg, vg, None, {(7, 5): configs[cc]})
+
+
+def test_flash_attention_data_parallel(fa):
+    """nn.DataParallel over the visible GPUs equals the direct call (tests/test_flash_attention_2.py:414-480)."""
+
+    class AttentionModel(torch.nn.Module):
+        def forward(self, q, k, v, scale):
+            return fa.flash_attention_v2(q, k, v, scale)
+
+    q, k, v, d_o = _seeded((4, 4, 256, 64), (4, 4, 256, 64), torch.float32)
+    scale = 0.125
+    ref = _run(fa, q, k, v, d_o, scale, False)
+    model = torch.nn.DataParallel(AttentionModel().cuda())
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = model(qg, kg, vg, scale)
+    out.backward(d_o.cuda())
+    for a, b in zip((out.detach(), qg.grad, kg.grad, vg.grad), ref):
+        assert torch.allclose(a, b, atol=1e-3, rtol=1e-3)
+
+
+# ------------------------------------------------------------------------- boundary behaviour on the device
+def test_non_contiguous_and_mixed_inputs(fa):
+    """Inputs are made contiguous and brought to one compute dtype like the reference does
+    (flash_attention_2.py:313-316); the output comes back in q's dtype."""
+    q, k, v, d_o = _seeded((2, 3, 160, 64), (2, 3, 160, 64), torch.float16)
+    want = oracle.naive_backward(q, k, v, d_o, None, torch.float32)
+    # (B, N, H, D) storage viewed as (B, H, N, D): non-contiguous
+    qn, kn, vn = (t.cuda().transpose(1, 2).contiguous().transpose(1, 2).requires_grad_(True) for t in (q, k, v))
+    assert not qn.is_contiguous()
+    out = fa.flash_attention_v2(qn, kn, vn)
+    out.backward(d_o.cuda().transpose(1, 2).contiguous().transpose(1, 2))
+    for name, g, w in zip(("o", "dq", "dk", "dv"), (out, qn.grad, kn.grad, vn.grad), want):
+        _assert_close(name, g, w)
+    # fp64 q with fp16 k, v: everything is computed in fp16, output in q's dtype
+    out64 = fa.flash_attention_v2(q.cuda().double(), k.cuda(), v.cuda())
+    assert out64.dtype == torch.float64
+    _assert_close("o (fp64 in)", out64, want[0])
+
+
+def test_zero_scale_means_default_and_explicit_scale_is_used(fa):
+    """`softmax_scale or default`: 0.0 selects 1/sqrt(D) (flash_attention_2.py:94)."""
+    q, k, v, _ = _seeded((1, 2, 96, 64), (1, 2, 96, 64), torch.bfloat16)
+    a = fa.flash_attention_v2(q.cuda(), k.cuda(), v.cuda(), 0.0)
+    b = fa.flash_attention_v2(q.cuda(), k.cuda(), v.cuda(), None)
+    assert torch.equal(a, b)
+    c = fa.flash_attention_v2(q.cuda(), k.cuda(), v.cuda(), 0.5)
+    _assert_close("o (scale 0.5)", c, oracle.naive_causal_attention(q, k, v, 0.5))
+
+
+def test_device_side_assertions(fa):
+    q = torch.zeros(1, 2, 16, 64, device="cuda", dtype=torch.float16)
+    with pytest.raises(AssertionError):
+        fa.flash_attention_v2(q, torch.zeros(1, 2, 16, 32, device="cuda", dtype=torch.float16), q)
+    big = torch.zeros(1, 1, 8, 160, device="cuda", dtype=torch.float16)
+    with pytest.raises(AssertionError, match="Supports head dimensions only up to"):
+        fa.flash_attention_v2(big, big, big)
