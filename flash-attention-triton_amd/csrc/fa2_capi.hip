@@ -99,15 +99,36 @@ int launch_status(const char *what) {
   return FA2_OK;
 }
 
+template <typename T, bool VEC>
+void launch_fwd_v(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
+  dim3 block(64 * fa2::kFwdWaves);
+  switch (dp) {
+    case 32: hipLaunchKernelGGL((fa2::fwd_kernel<T, 32, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
+    case 64: hipLaunchKernelGGL((fa2::fwd_kernel<T, 64, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
+    case 96: hipLaunchKernelGGL((fa2::fwd_kernel<T, 96, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fa2::fwd_kernel<T, 128, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
+  }
+}
+
+// The fast kernels need the exact padded head dimension, 16-byte aligned rows and row offsets
+// inside a tile that fit 32 bits.
+bool direct_ok(const fa2::Tensor4 &t) { return t.stride_seq < (int64_t(1) << 24); }
+
 template <typename T>
 void launch_fwd(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
   dim3 block(64 * fa2::kFwdWaves);
-  switch (dp) {
-    case 32: hipLaunchKernelGGL((fa2::fwd_kernel<T, 32, kFwdBlockKV>), grid, block, 0, s, p); break;
-    case 64: hipLaunchKernelGGL((fa2::fwd_kernel<T, 64, kFwdBlockKV>), grid, block, 0, s, p); break;
-    case 96: hipLaunchKernelGGL((fa2::fwd_kernel<T, 96, kFwdBlockKV>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fa2::fwd_kernel<T, 128, kFwdBlockKV>), grid, block, 0, s, p); break;
+  if (p.vec && p.headdim == dp && dp != 96 && direct_ok(p.k) && direct_ok(p.v)) {
+    switch (dp) {
+      case 32: hipLaunchKernelGGL((fa2::fwd_direct_kernel<T, 32, kFwdBlockKV>), grid, block, 0, s, p); break;
+      case 64: hipLaunchKernelGGL((fa2::fwd_direct_kernel<T, 64, kFwdBlockKV>), grid, block, 0, s, p); break;
+      default: hipLaunchKernelGGL((fa2::fwd_direct_kernel<T, 128, kFwdBlockKV>), grid, block, 0, s, p); break;
+    }
+    return;
   }
+  if (p.vec)
+    launch_fwd_v<T, true>(dp, p, grid, s);
+  else
+    launch_fwd_v<T, false>(dp, p, grid, s);
 }
 
 template <typename T>

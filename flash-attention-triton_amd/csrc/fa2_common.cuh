@@ -177,3 +177,82 @@ __device__ __forceinline__ void store_transposed_acc(const f32x16 (&acc)[DP / 32
 }
 
 }  // namespace fa2
+
+// ------------------------------------------------------------------------------------------
+// Swizzled, unpadded LDS tiles filled by LDS-direct global loads.
+//
+// A tile of R rows x DP halves is stored with row pitch DP (no padding).  A row holds DP/8
+// 16-byte chunks; logical chunk c of row r lives in slot c ^ swz<DP>(r).  The swizzle is chosen
+// so that, on the 64-bank LDS of gfx950, both access patterns used by the kernels are free of
+// bank conflicts:
+//   * 16-byte row reads (ds_read_b128): 16 consecutive rows, same logical chunk;
+//   * transposing reads (ds_read_b64_tr_b16): 4 consecutive rows x 4 consecutive chunks.
+// global_load_lds_dwordx4 writes lane l's 16 bytes at (wave-uniform LDS base) + 16*l, so one
+// wave-load fills 1 KiB of consecutive slots; the swizzle is applied on the global-address side
+// (slot s of row r is loaded from chunk s ^ swz(r)).
+// ------------------------------------------------------------------------------------------
+template <int DP>
+__device__ __forceinline__ int swz(int r);
+template <>
+__device__ __forceinline__ int swz<128>(int r) { return 4 * (r & 3) + ((r >> 2) & 3); }
+template <>
+__device__ __forceinline__ int swz<64>(int r) { return 4 * ((r >> 1) & 1) + ((r >> 2) & 3); }
+template <>
+__device__ __forceinline__ int swz<32>(int r) { return (r >> 2) & 3; }
+
+// Element offset of (row r, logical chunk c) in a swizzled tile.
+template <int DP>
+__device__ __forceinline__ int swz_off(int r, int c) { return r * DP + ((c ^ swz<DP>(r)) << 3); }
+
+__device__ __forceinline__ void load_lds_16(const short *gsrc, short *lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gsrc,
+                                   (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
+}
+
+// Streams ROWS x DP tiles of a (seqlen, headdim) matrix into swizzled LDS with LDS-direct loads.
+// All NW waves of the workgroup take part; each wave issues LOADS loads of 1 KiB per tile.
+template <int DP, int ROWS, int NW>
+struct TileLoader {
+  static constexpr int CPR = DP / 8;    // chunks per row
+  static constexpr int RPL = 64 / CPR;  // rows per wave-load
+  static constexpr int NL = ROWS / RPL; // wave-loads per tile
+  static constexpr int LOADS = NL / NW; // per wave
+  static_assert(NL % NW == 0 && LOADS >= 1, "tile must split evenly over the waves");
+  // Multiples of NW*RPL rows keep the low four row bits the swizzle looks at, so a lane's
+  // swizzled chunk does not depend on the load index.
+  static_assert((NW * RPL) % 16 == 0, "swizzle must be independent of the load index");
+  static constexpr int TILE_ELEMS = ROWS * DP;
+
+  const short *base;  // first row of the matrix for this (batch, head)
+  int64_t stride;     // row stride in elements
+  int wave;
+  int row_in;         // this lane's row within the tile for load 0
+  int chunk;          // this lane's global chunk index
+  unsigned voff;      // element offset of this lane inside a tile for load 0
+
+  __device__ __forceinline__ TileLoader(const short *base_, int64_t stride_) : base(base_), stride(stride_) {
+    const int lane = threadIdx.x & 63;
+    wave = threadIdx.x >> 6;
+    row_in = wave * RPL + lane / CPR;
+    chunk = (lane % CPR) ^ swz<DP>(row_in);
+    voff = (unsigned)(row_in * (int)stride + chunk * 8);
+  }
+
+  // Rows [row0, row0 + ROWS), all inside the matrix -> tile at `lds`.
+  __device__ __forceinline__ void issue(int row0, short *lds) const {
+    const short *tile = base + (int64_t)row0 * stride;
+#pragma unroll
+    for (int i = 0; i < LOADS; i++)
+      load_lds_16(tile + (int64_t)(i * NW * RPL) * stride + voff, lds + (i * NW + wave) * 512);
+  }
+
+  // Same, but rows at or beyond `nrows` are taken from row nrows - 1 (finite values that the
+  // caller masks).
+  __device__ __forceinline__ void issue_clamped(int row0, int nrows, short *lds) const {
+#pragma unroll
+    for (int i = 0; i < LOADS; i++) {
+      const int r = min(row0 + i * NW * RPL + row_in, nrows - 1);
+      load_lds_16(base + (int64_t)r * stride + chunk * 8, lds + (i * NW + wave) * 512);
+    }
+  }
+};

@@ -17,8 +17,8 @@
 //  * Unlike the reference (mask applied to every tile, lines 139-147) the mask is evaluated only
 //    on tiles that touch the diagonal or the end of the key sequence, and sub-blocks entirely
 //    above the diagonal are skipped.
-//  * The running maximum `m` is the usual one; the reference floors it with the running lse
-//    (line 150), which only changes rounding.
+//  * The maximum the probabilities are formed against is raised lazily (see kRescaleSlack); the
+//    reference floors its maximum with the running lse (line 150).  Both only change rounding.
 #pragma once
 
 #include "fa2_common.cuh"
@@ -38,10 +38,16 @@ struct FwdParams {
 constexpr int kFwdWaves = 4;
 constexpr int kFwdBlockQ = 32 * kFwdWaves;
 
+// The running max is only raised (and the accumulator rescaled) when some row's new maximum
+// exceeds the one in use by more than this many powers of two; until then probabilities are
+// formed against the stale maximum and may reach 2^kRescaleSlack, which fp32 sums and bf16/fp16
+// operands hold without loss.  The final division by the row sum removes the common factor.
+constexpr float kRescaleSlack = 8.0f;
+
 template <int DP, int BKV>
 struct FwdLayout {
-  static constexpr int KLD = DP + 8;   // K tile row pitch: conflict-free 16-byte row reads
-  static constexpr int VLD = DP + 8;   // V tile row pitch (read with transposing loads)
+  static constexpr int KLD = DP + 8;    // K tile row pitch: conflict-free 16-byte row reads
+  static constexpr int VLD = DP + 32;   // V tile row pitch: conflict-free transposing reads
   static constexpr int K_ELEMS = BKV * KLD;
   static constexpr int V_ELEMS = BKV * VLD;
   static constexpr int STAGE_ELEMS = K_ELEMS + V_ELEMS;
@@ -50,13 +56,90 @@ struct FwdLayout {
       (2 * STAGE_ELEMS > PATCH_ELEMS) ? 2 * STAGE_ELEMS : PATCH_ELEMS;
 };
 
-template <typename T, int DP, int BKV>
+// One key/value tile for one wave: S^T = K Q^T, online softmax, O^T += V^T P^T.
+// MASKED tiles apply the causal and key-length masks element by element.
+template <typename T, int DP, int BKV, bool MASKED>
+__device__ __forceinline__ void fwd_tile(const short *sk, const short *sv, const s16x8 (&qf)[DP / 16],
+                                         f32x16 (&oacc)[DP / 32], float &m_ref, float &l_run,
+                                         float scale_log2, int kvt, int qrow, int seqlen_k,
+                                         int k_frag_off, int v_frag_off) {
+  using L = FwdLayout<DP, BKV>;
+  constexpr int KS = DP / 16, DB = DP / 32, MB = BKV / 32, KS2 = BKV / 16;
+  const int h = (threadIdx.x >> 5) & 1;
+
+  f32x16 s[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++) {
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    s[mb] = zero;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      s16x8 a = *reinterpret_cast<const s16x8 *>(sk + k_frag_off + 32 * mb * L::KLD + 16 * ks);
+      s[mb] = Elem<T>::mfma(a, qf[ks], s[mb]);
+    }
+  }
+  if (MASKED) {
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int kv = kvt + 32 * mb + 8 * (i >> 2) + 4 * h + (i & 3);
+        if (kv > qrow || kv >= seqlen_k) s[mb][i] = -INFINITY;
+      }
+  }
+
+  float mloc = s[0][0];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) mloc = fmaxf(mloc, s[mb][i]);
+  mloc = max_over_halves(mloc);
+
+  // Raise the reference maximum only when some row needs it (wave-uniform branch).
+  const bool grow = (mloc - m_ref) * scale_log2 > kRescaleSlack;  // true on the first tile (m_ref = -inf)
+  if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+    const float m_new = fmaxf(m_ref, mloc);
+    // Every query column of a processed tile sees at least key kvt, so m_new is finite.
+    const float alpha = fast_exp2((m_ref - m_new) * scale_log2);
+    m_ref = m_new;
+    l_run *= alpha;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+  }
+  const float mc = m_ref * scale_log2;
+
+  s16x8 pf[KS2];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++) {
+    f32x16 e;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      e[i] = fast_exp2(s[mb][i] * scale_log2 - mc);
+      l_run += e[i];
+    }
+    f32x8 lo = {e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]};
+    f32x8 hi = {e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]};
+    pf[2 * mb] = Elem<T>::pack8(lo);
+    pf[2 * mb + 1] = Elem<T>::pack8(hi);
+  }
+
+#pragma unroll
+  for (int ks2 = 0; ks2 < KS2; ks2++) {
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      s16x8 a = lds_read_tr_frag(sv + v_frag_off + 16 * ks2 * L::VLD + 32 * db, L::VLD);
+      oacc[db] = Elem<T>::mfma(a, pf[ks2], oacc[db]);
+    }
+  }
+}
+
+template <typename T, int DP, int BKV, bool VEC>
 __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams p) {
   using L = FwdLayout<DP, BKV>;
   constexpr int KS = DP / 16;    // k-steps of Q K^T
   constexpr int DB = DP / 32;    // 32-row blocks of O^T
-  constexpr int MB = BKV / 32;   // 32-row blocks of S^T
-  constexpr int KS2 = BKV / 16;  // k-steps of P V
   constexpr int CPR = DP / 8;    // 16-byte chunks per tile row
   constexpr int NTHREADS = 64 * kFwdWaves;
   constexpr int CPT = (BKV * CPR) / NTHREADS;  // chunks per thread per tile
@@ -78,7 +161,6 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams 
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int q0 = qt * kFwdBlockQ;
   const int q0w = q0 + 32 * wave;
-  const bool vec = p.vec != 0;
 
   const short *Q = (const short *)p.q.ptr + b * p.q.stride_batch + hd * p.q.stride_head;
   const short *K = (const short *)p.k.ptr + b * p.k.stride_batch + hd * p.k.stride_head;
@@ -93,11 +175,14 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams 
     const bool ok = row < p.seqlen_q;
     const short *rp = Q + (int64_t)row * p.q.stride_seq;
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[ks] = load_chunk(rp, 16 * ks + 8 * h, p.headdim, ok, vec);
+    for (int ks = 0; ks < KS; ks++) qf[ks] = load_chunk(rp, 16 * ks + 8 * h, p.headdim, ok, VEC);
   }
 
   const int kv_end = min(q0 + kFwdBlockQ, p.seqlen_k);
   const int n_tiles = (kv_end + BKV - 1) / BKV;
+  // Leading tiles that lie entirely at or below this wave's first query row and inside the key
+  // range need no mask; tiles starting beyond the wave's last row are skipped.
+  const int n_full = max(0, min(min(q0w + 1, p.seqlen_k) / BKV, n_tiles));
 
   s16x8 kreg[CPT], vreg[CPT];
   auto load_tile = [&](int kvt) {
@@ -107,8 +192,8 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams 
       const int r = id / CPR, cc = id % CPR;
       const int kv = kvt + r;
       const bool ok = kv < p.seqlen_k;
-      kreg[i] = load_chunk(K + (int64_t)kv * p.k.stride_seq, cc * 8, p.headdim, ok, vec);
-      vreg[i] = load_chunk(V + (int64_t)kv * p.v.stride_seq, cc * 8, p.headdim, ok, vec);
+      kreg[i] = load_chunk(K + (int64_t)kv * p.k.stride_seq, cc * 8, p.headdim, ok, VEC);
+      vreg[i] = load_chunk(V + (int64_t)kv * p.v.stride_seq, cc * 8, p.headdim, ok, VEC);
     }
   };
   auto store_tile = [&](int buf) {
@@ -128,7 +213,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams 
   for (int db = 0; db < DB; db++)
 #pragma unroll
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
-  float m_run = -INFINITY;  // running max of the raw (unscaled) scores of this lane's query
+  float m_ref = -INFINITY;  // maximum (raw, unscaled scores) the probabilities are formed against
   float l_run = 0.f;        // this lane's share of the running sum (its half of the key rows)
 
   load_tile(0);
@@ -136,8 +221,9 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams 
   __syncthreads();
 
   // Per-lane LDS offsets that do not depend on the tile.
-  const int k_frag_off = c * L::KLD + 8 * h;                                  // + 32mb*KLD + 16ks
+  const int k_frag_off = c * L::KLD + 8 * h;                                       // + 32mb*KLD + 16ks
   const int v_frag_off = (4 * h + (i16 >> 2)) * L::VLD + 16 * g2 + 4 * (i16 & 3);  // + 16ks2*VLD + 32db
+  const int qrow = q0w + c;
 
   for (int t = 0; t < n_tiles; t++) {
     const int buf = t & 1;
@@ -145,91 +231,14 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams 
     const bool more = (t + 1) < n_tiles;
     if (more) load_tile(kvt + BKV);
 
-    // Key sub-blocks (32 rows) of this tile that reach this wave's query range at all.
-    int nact = (q0w + 31 - kvt) / 32 + 1;
-    nact = (q0w + 31 < kvt) ? 0 : min(nact, MB);
-
-    if (nact > 0) {
-      const short *sk = smem + buf * L::STAGE_ELEMS;
-      const short *sv = sk + L::K_ELEMS;
-
-      f32x16 s[MB];
-#pragma unroll
-      for (int mb = 0; mb < MB; mb++) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) s[mb][i] = 0.f;
-        if (mb < nact) {
-#pragma unroll
-          for (int ks = 0; ks < KS; ks++) {
-            s16x8 a = *reinterpret_cast<const s16x8 *>(sk + k_frag_off + 32 * mb * L::KLD + 16 * ks);
-            s[mb] = Elem<T>::mfma(a, qf[ks], s[mb]);
-          }
-        }
-      }
-
-      // Mask: needed when the tile crosses the diagonal of this wave's rows or the key end.
-      const bool need_mask = (kvt + 32 * nact - 1 > q0w) || (kvt + 32 * nact > p.seqlen_k);
-      if (need_mask) {
-        const int qrow = q0w + c;
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const int kv = kvt + 32 * mb + 8 * (i >> 2) + 4 * h + (i & 3);
-            if (kv > qrow || kv >= p.seqlen_k) s[mb][i] = -INFINITY;
-          }
-      }
-#pragma unroll
-      for (int mb = 0; mb < MB; mb++)
-        if (mb >= nact) {
-#pragma unroll
-          for (int i = 0; i < 16; i++) s[mb][i] = -INFINITY;
-        }
-
-      float mloc = -INFINITY;
-#pragma unroll
-      for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) mloc = fmaxf(mloc, s[mb][i]);
-      mloc = max_over_halves(mloc);
-      const float m_new = fmaxf(m_run, mloc);
-      // Every query column of an active tile sees at least key kvt, so m_new is finite here.
-      const float mc = m_new * p.scale_log2;
-      const float alpha = fast_exp2(m_run * p.scale_log2 - mc);
-      m_run = m_new;
-
-      float lsum = 0.f;
-      s16x8 pf[KS2];
-#pragma unroll
-      for (int mb = 0; mb < MB; mb++) {
-        f32x16 e;
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          e[i] = fast_exp2(s[mb][i] * p.scale_log2 - mc);
-          lsum += e[i];
-        }
-        f32x8 lo = {e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]};
-        f32x8 hi = {e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]};
-        pf[2 * mb] = Elem<T>::pack8(lo);
-        pf[2 * mb + 1] = Elem<T>::pack8(hi);
-      }
-      l_run = l_run * alpha + lsum;
-
-#pragma unroll
-      for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
-
-#pragma unroll
-      for (int ks2 = 0; ks2 < KS2; ks2++) {
-        if ((ks2 >> 1) < nact) {
-#pragma unroll
-          for (int db = 0; db < DB; db++) {
-            s16x8 a = lds_read_tr_frag(sv + v_frag_off + 16 * ks2 * L::VLD + 32 * db, L::VLD);
-            oacc[db] = Elem<T>::mfma(a, pf[ks2], oacc[db]);
-          }
-        }
-      }
+    const short *sk = smem + buf * L::STAGE_ELEMS;
+    const short *sv = sk + L::K_ELEMS;
+    if (t < n_full) {
+      fwd_tile<T, DP, BKV, false>(sk, sv, qf, oacc, m_ref, l_run, p.scale_log2, kvt, qrow,
+                                  p.seqlen_k, k_frag_off, v_frag_off);
+    } else if (kvt <= q0w + 31) {
+      fwd_tile<T, DP, BKV, true>(sk, sv, qf, oacc, m_ref, l_run, p.scale_log2, kvt, qrow,
+                                 p.seqlen_k, k_frag_off, v_frag_off);
     }
 
     if (more) store_tile(buf ^ 1);
@@ -239,14 +248,222 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams 
   // Epilogue: normalise, write lse and O.
   const float l_tot = sum_over_halves(l_run);
   const float inv_l = 1.f / l_tot;
-  if (h == 0 && q0w + c < p.seqlen_q) LSE[q0w + c] = m_run * p.scale + __logf(l_tot);
+  if (h == 0 && q0w + c < p.seqlen_q) LSE[q0w + c] = m_ref * p.scale + __logf(l_tot);
   if (qt == p.n_qtiles - 1) {
     for (int r = p.seqlen_q + tid; r < p.seqlen_q_rounded; r += NTHREADS) LSE[r] = 0.f;
   }
   // All waves passed the loop's final barrier, so the K/V stages are free to reuse.
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(oacc, inv_l, patch, O + (int64_t)q0w * p.o.stride_seq,
-                              p.o.stride_seq, p.seqlen_q - q0w, p.headdim, vec);
+                              p.o.stride_seq, p.seqlen_q - q0w, p.headdim, VEC);
+}
+
+// ------------------------------------------------------------------------------------------
+// Fast path: head dimension equal to the padded one and 16-byte aligned rows.  K and V tiles go
+// straight from global memory into swizzled, unpadded LDS (no staging registers, no LDS stores),
+// two stages deep; everything else is as in fwd_kernel.
+// ------------------------------------------------------------------------------------------
+template <int DP, int BKV>
+struct FwdDirectLayout {
+  static constexpr int TILE_ELEMS = BKV * DP;
+  static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;  // K tile then V tile
+  static constexpr int STAGES = 2;
+  static constexpr int PATCH_ELEMS = kFwdWaves * 32 * (DP + 8);
+  static constexpr int TOTAL_ELEMS =
+      (STAGES * STAGE_ELEMS > PATCH_ELEMS) ? STAGES * STAGE_ELEMS : PATCH_ELEMS;
+};
+
+// s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt fields left at their maxima).
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+template <typename T, int DP, int BKV, bool MASKED>
+__device__ __forceinline__ void fwd_tile_direct(const short *sk, const short *sv,
+                                                const s16x8 (&qf)[DP / 16], f32x16 (&oacc)[DP / 32],
+                                                float &m_ref, float &l_run, float scale_log2,
+                                                int kvt, int qrow, int seqlen_k,
+                                                const int (&kaddr)[DP / 16],
+                                                const int (&valo)[DP / 32],
+                                                const int (&vahi)[DP / 32]) {
+  constexpr int KS = DP / 16, DB = DP / 32, MB = BKV / 32, KS2 = BKV / 16;
+  const int h = (threadIdx.x >> 5) & 1;
+
+  f32x16 s[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++) {
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    s[mb] = zero;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      s16x8 a = *reinterpret_cast<const s16x8 *>(sk + kaddr[ks] + 32 * mb * DP);
+      s[mb] = Elem<T>::mfma(a, qf[ks], s[mb]);
+    }
+  }
+  if (MASKED) {
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int kv = kvt + 32 * mb + 8 * (i >> 2) + 4 * h + (i & 3);
+        if (kv > qrow || kv >= seqlen_k) s[mb][i] = -INFINITY;
+      }
+  }
+
+  float mloc = s[0][0];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) mloc = fmaxf(mloc, s[mb][i]);
+  mloc = max_over_halves(mloc);
+
+  const bool grow = (mloc - m_ref) * scale_log2 > kRescaleSlack;
+  if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+    const float m_new = fmaxf(m_ref, mloc);
+    const float alpha = fast_exp2((m_ref - m_new) * scale_log2);
+    m_ref = m_new;
+    l_run *= alpha;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+  }
+  const float mc = m_ref * scale_log2;
+
+  s16x8 pf[KS2];
+#pragma unroll
+  for (int mb = 0; mb < MB; mb++) {
+    f32x16 e;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      e[i] = fast_exp2(s[mb][i] * scale_log2 - mc);
+      l_run += e[i];
+    }
+    f32x8 lo = {e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]};
+    f32x8 hi = {e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]};
+    pf[2 * mb] = Elem<T>::pack8(lo);
+    pf[2 * mb + 1] = Elem<T>::pack8(hi);
+  }
+
+#pragma unroll
+  for (int ks2 = 0; ks2 < KS2; ks2++) {
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      s16x4 lo = lds_read_tr(sv + valo[db] + 16 * ks2 * DP);
+      s16x4 hi = lds_read_tr(sv + vahi[db] + 16 * ks2 * DP);
+      s16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      oacc[db] = Elem<T>::mfma(a, pf[ks2], oacc[db]);
+    }
+  }
+}
+
+template <typename T, int DP, int BKV>
+__global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const FwdParams p) {
+  using L = FwdDirectLayout<DP, BKV>;
+  constexpr int KS = DP / 16, DB = DP / 32;
+  constexpr int NTHREADS = 64 * kFwdWaves;
+
+  __shared__ __attribute__((aligned(1024))) short smem[L::TOTAL_ELEMS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 31, h = lane >> 5;
+  const int i16 = lane & 15, g2 = (lane >> 4) & 1;
+
+  const int BH = p.batch * p.nheads;
+  const int bh = blockIdx.x % BH;
+  const int qt = p.n_qtiles - 1 - blockIdx.x / BH;
+  const int b = bh / p.nheads, hd = bh % p.nheads;
+  const int q0 = qt * kFwdBlockQ;
+  const int q0w = q0 + 32 * wave;
+
+  const short *Q = (const short *)p.q.ptr + b * p.q.stride_batch + hd * p.q.stride_head;
+  const short *K = (const short *)p.k.ptr + b * p.k.stride_batch + hd * p.k.stride_head;
+  const short *V = (const short *)p.v.ptr + b * p.v.stride_batch + hd * p.v.stride_head;
+  short *O = (short *)p.o.ptr + b * p.o.stride_batch + hd * p.o.stride_head;
+  float *LSE = p.lse + (int64_t)bh * p.seqlen_q_rounded;
+
+  const TileLoader<DP, BKV, kFwdWaves> kload(K, p.k.stride_seq), vload(V, p.v.stride_seq);
+
+  const int kv_end = min(q0 + kFwdBlockQ, p.seqlen_k);
+  const int n_tiles = (kv_end + BKV - 1) / BKV;
+  const int n_full = max(0, min(min(q0w + 1, p.seqlen_k) / BKV, n_tiles));
+  const int n_inside = p.seqlen_k / BKV;  // tiles whose every row exists
+
+  auto issue_tile = [&](int t) {
+    short *stage = smem + (t & 1) * L::STAGE_ELEMS;
+    if (t < n_inside) {
+      kload.issue(t * BKV, stage);
+      vload.issue(t * BKV, stage + L::TILE_ELEMS);
+    } else {
+      kload.issue_clamped(t * BKV, p.seqlen_k, stage);
+      vload.issue_clamped(t * BKV, p.seqlen_k, stage + L::TILE_ELEMS);
+    }
+  };
+  issue_tile(0);
+
+  // Q^T fragments (B operand of S^T = K Q^T): lane (c, h) holds Q[q0w + c][16 ks + 8 h + j].
+  s16x8 qf[KS];
+  {
+    const int row = q0w + c;
+    const bool ok = row < p.seqlen_q;
+    const short *rp = Q + (int64_t)row * p.q.stride_seq;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = load_chunk(rp, 16 * ks + 8 * h, DP, ok, true);
+  }
+
+  // Fragment offsets inside a tile (swizzled); tile-relative row blocks are added as immediates.
+  int kaddr[KS], valo[DB], vahi[DB];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) kaddr[ks] = swz_off<DP>(c, 2 * ks + h);
+  {
+    const int rowlo = 4 * h + (i16 >> 2);
+    const int sub = (i16 & 1) * 4;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      const int chunk = 4 * db + 2 * g2 + ((i16 & 3) >> 1);
+      valo[db] = swz_off<DP>(rowlo, chunk) + sub;
+      vahi[db] = swz_off<DP>(rowlo + 8, chunk) + sub;
+    }
+  }
+
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
+  float m_ref = -INFINITY;
+  float l_run = 0.f;
+  const int qrow = q0w + c;
+
+  wait_vmem_all();
+  __syncthreads();
+
+  for (int t = 0; t < n_tiles; t++) {
+    const int kvt = t * BKV;
+    if (t + 1 < n_tiles) issue_tile(t + 1);
+
+    const short *sk = smem + (t & 1) * L::STAGE_ELEMS;
+    const short *sv = sk + L::TILE_ELEMS;
+    if (t < n_full) {
+      fwd_tile_direct<T, DP, BKV, false>(sk, sv, qf, oacc, m_ref, l_run, p.scale_log2, kvt, qrow,
+                                         p.seqlen_k, kaddr, valo, vahi);
+    } else if (kvt <= q0w + 31) {
+      fwd_tile_direct<T, DP, BKV, true>(sk, sv, qf, oacc, m_ref, l_run, p.scale_log2, kvt, qrow,
+                                        p.seqlen_k, kaddr, valo, vahi);
+    }
+
+    wait_vmem_all();
+    __syncthreads();
+  }
+
+  const float l_tot = sum_over_halves(l_run);
+  const float inv_l = 1.f / l_tot;
+  if (h == 0 && q0w + c < p.seqlen_q) LSE[q0w + c] = m_ref * p.scale + __logf(l_tot);
+  if (qt == p.n_qtiles - 1) {
+    for (int r = p.seqlen_q + tid; r < p.seqlen_q_rounded; r += NTHREADS) LSE[r] = 0.f;
+  }
+  short *patch = smem + wave * 32 * (DP + 8);
+  store_transposed_acc<T, DP>(oacc, inv_l, patch, O + (int64_t)q0w * p.o.stride_seq,
+                              p.o.stride_seq, p.seqlen_q - q0w, DP, true);
 }
 
 }  // namespace fa2
