@@ -56,6 +56,12 @@ struct Elem<__bf16> {
   static __device__ __forceinline__ float to_float(short x) {
     return __builtin_bit_cast(float, ((unsigned)(unsigned short)x) << 16);
   }
+  // acc + lo(pair) + hi(pair) for a packed pair of values (v_dot2c_f32_bf16 with a vector of ones).
+  static __device__ __forceinline__ float add_pair(unsigned pair, float acc) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair), ones, acc, false);
+  }
 };
 
 template <>
@@ -72,6 +78,11 @@ struct Elem<_Float16> {
   }
   static __device__ __forceinline__ float to_float(short x) {
     return (float)__builtin_bit_cast(_Float16, x);
+  }
+  static __device__ __forceinline__ float add_pair(unsigned pair, float acc) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pair), ones, acc, false);
   }
 };
 
@@ -204,9 +215,34 @@ __device__ __forceinline__ int swz<32>(int r) { return (r >> 2) & 3; }
 template <int DP>
 __device__ __forceinline__ int swz_off(int r, int c) { return r * DP + ((c ^ swz<DP>(r)) << 3); }
 
+// LDS-direct load of 16 bytes per lane: lane l's data lands at lds_wave_base + 16*l.
+// Written as inline assembly on purpose: with the compiler builtin every later LDS read is made
+// to wait for the load (the compiler cannot tell which LDS bytes the DMA writes), which would
+// serialise the prefetch.  The callers order these loads against LDS reads themselves with
+// `s_waitcnt vmcnt(0)` followed by a workgroup barrier.
 __device__ __forceinline__ void load_lds_16(const short *gsrc, short *lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gsrc,
-                                   (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
+  const unsigned lds_addr =
+      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base;
+  asm volatile(
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, off"
+      :
+      : "v"(gsrc), "s"(lds_addr)
+      : "memory");
+}
+// Same with the address split into a wave-uniform base (SGPR pair) and a per-lane byte offset.
+__device__ __forceinline__ void load_lds_16(const short *uniform_base, unsigned lane_byte_offset,
+                                            short *lds_wave_base) {
+  const unsigned lds_addr =
+      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base;
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %1"
+      :
+      : "v"(lane_byte_offset), "s"(uniform_base), "s"(lds_addr)
+      : "memory");
 }
 
 // Streams ROWS x DP tiles of a (seqlen, headdim) matrix into swizzled LDS with LDS-direct loads.
@@ -228,14 +264,14 @@ struct TileLoader {
   int wave;
   int row_in;         // this lane's row within the tile for load 0
   int chunk;          // this lane's global chunk index
-  unsigned voff;      // element offset of this lane inside a tile for load 0
+  unsigned voff;      // byte offset of this lane inside a tile for load 0
 
   __device__ __forceinline__ TileLoader(const short *base_, int64_t stride_) : base(base_), stride(stride_) {
     const int lane = threadIdx.x & 63;
-    wave = threadIdx.x >> 6;
+    wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     row_in = wave * RPL + lane / CPR;
     chunk = (lane % CPR) ^ swz<DP>(row_in);
-    voff = (unsigned)(row_in * (int)stride + chunk * 8);
+    voff = 2u * (unsigned)(row_in * (int)stride + chunk * 8);
   }
 
   // Rows [row0, row0 + ROWS), all inside the matrix -> tile at `lds`.
@@ -243,7 +279,7 @@ struct TileLoader {
     const short *tile = base + (int64_t)row0 * stride;
 #pragma unroll
     for (int i = 0; i < LOADS; i++)
-      load_lds_16(tile + (int64_t)(i * NW * RPL) * stride + voff, lds + (i * NW + wave) * 512);
+      load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (i * NW + wave) * 512);
   }
 
   // Same, but rows at or beyond `nrows` are taken from row nrows - 1 (finite values that the

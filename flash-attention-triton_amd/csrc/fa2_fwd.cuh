@@ -21,6 +21,8 @@
 //    reference floors its maximum with the running lse (line 150).  Both only change rounding.
 #pragma once
 
+#include <type_traits>
+
 #include "fa2_common.cuh"
 
 namespace fa2 {
@@ -259,112 +261,56 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams 
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast path: head dimension equal to the padded one and 16-byte aligned rows.  K and V tiles go
-// straight from global memory into swizzled, unpadded LDS (no staging registers, no LDS stores),
-// two stages deep; everything else is as in fwd_kernel.
+// Fast path: head dimension equal to the padded one and 16-byte aligned rows.
+//
+//  * K and V tiles go straight from global memory into swizzled, unpadded LDS
+//    (global_load_lds_dwordx4: no staging registers, no LDS stores), two stages each.
+//  * One workgroup barrier per tile, placed between the two GEMMs.  At that point every wave has
+//    finished reading K_t and V_{t-1}, so K_{t+2} and V_{t+1} are issued right after it and have
+//    a whole tile of time to land.
+//  * MFMA operand fragments travel through a ring of DP/16 registers-sets that is always loaded
+//    ahead of use: while S^T block 0 is multiplied the ring refills with block 1; V^T fragments
+//    are fetched before the softmax arithmetic starts; the tail of the P V GEMM refills the ring
+//    with the next tile's first K fragments.  LDS latency is therefore never waited for.
 // ------------------------------------------------------------------------------------------
 template <int DP, int BKV>
 struct FwdDirectLayout {
   static constexpr int TILE_ELEMS = BKV * DP;
-  static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;  // K tile then V tile
-  static constexpr int STAGES = 2;
+  static constexpr int K_BASE = 0;                 // two K stages
+  static constexpr int V_BASE = 2 * TILE_ELEMS;    // two V stages
   static constexpr int PATCH_ELEMS = kFwdWaves * 32 * (DP + 8);
-  static constexpr int TOTAL_ELEMS =
-      (STAGES * STAGE_ELEMS > PATCH_ELEMS) ? STAGES * STAGE_ELEMS : PATCH_ELEMS;
+  static constexpr int TOTAL_ELEMS = (4 * TILE_ELEMS > PATCH_ELEMS) ? 4 * TILE_ELEMS : PATCH_ELEMS;
 };
 
 // s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt fields left at their maxima).
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-template <typename T, int DP, int BKV, bool MASKED>
-__device__ __forceinline__ void fwd_tile_direct(const short *sk, const short *sv,
-                                                const s16x8 (&qf)[DP / 16], f32x16 (&oacc)[DP / 32],
-                                                float &m_ref, float &l_run, float scale_log2,
-                                                int kvt, int qrow, int seqlen_k,
-                                                const int (&kaddr)[DP / 16],
-                                                const int (&valo)[DP / 32],
-                                                const int (&vahi)[DP / 32]) {
-  constexpr int KS = DP / 16, DB = DP / 32, MB = BKV / 32, KS2 = BKV / 16;
-  const int h = (threadIdx.x >> 5) & 1;
-
-  f32x16 s[MB];
-#pragma unroll
-  for (int mb = 0; mb < MB; mb++) {
-    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    s[mb] = zero;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      s16x8 a = *reinterpret_cast<const s16x8 *>(sk + kaddr[ks] + 32 * mb * DP);
-      s[mb] = Elem<T>::mfma(a, qf[ks], s[mb]);
-    }
-  }
-  if (MASKED) {
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        const int kv = kvt + 32 * mb + 8 * (i >> 2) + 4 * h + (i & 3);
-        if (kv > qrow || kv >= seqlen_k) s[mb][i] = -INFINITY;
-      }
-  }
-
-  float mloc = s[0][0];
-#pragma unroll
-  for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) mloc = fmaxf(mloc, s[mb][i]);
-  mloc = max_over_halves(mloc);
-
-  const bool grow = (mloc - m_ref) * scale_log2 > kRescaleSlack;
-  if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-    const float m_new = fmaxf(m_ref, mloc);
-    const float alpha = fast_exp2((m_ref - m_new) * scale_log2);
-    m_ref = m_new;
-    l_run *= alpha;
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
-  }
-  const float mc = m_ref * scale_log2;
-
-  s16x8 pf[KS2];
-#pragma unroll
-  for (int mb = 0; mb < MB; mb++) {
-    f32x16 e;
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-      e[i] = fast_exp2(s[mb][i] * scale_log2 - mc);
-      l_run += e[i];
-    }
-    f32x8 lo = {e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]};
-    f32x8 hi = {e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]};
-    pf[2 * mb] = Elem<T>::pack8(lo);
-    pf[2 * mb + 1] = Elem<T>::pack8(hi);
-  }
-
-#pragma unroll
-  for (int ks2 = 0; ks2 < KS2; ks2++) {
-#pragma unroll
-    for (int db = 0; db < DB; db++) {
-      s16x4 lo = lds_read_tr(sv + valo[db] + 16 * ks2 * DP);
-      s16x4 hi = lds_read_tr(sv + vahi[db] + 16 * ks2 * DP);
-      s16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      oacc[db] = Elem<T>::mfma(a, pf[ks2], oacc[db]);
-    }
-  }
-}
+#ifdef FA2_PHASE_TIMING
+// Debug build only: cycles spent in each phase, summed over tiles, for workgroup 0's waves.
+__device__ long long fa2_phase_cycles[8][8];
+__device__ long long fa2_wg_times[8192][4];
+#define FA2_TICK(slot)                                        \
+  do {                                                        \
+    const long long now_ = __builtin_amdgcn_s_memtime();      \
+    if (blockIdx.x == FA2_PHASE_TIMING) phase_acc[slot] += now_ - tick_; \
+    tick_ = now_;                                             \
+  } while (0)
+#else
+#define FA2_TICK(slot) do {} while (0)
+#endif
 
 template <typename T, int DP, int BKV>
 __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const FwdParams p) {
   using L = FwdDirectLayout<DP, BKV>;
-  constexpr int KS = DP / 16, DB = DP / 32;
+  constexpr int KS = DP / 16, DB = DP / 32, MB = BKV / 32, KS2 = BKV / 16;
   constexpr int NTHREADS = 64 * kFwdWaves;
+  static_assert(MB == 2 && KS2 == 4 && KS == 2 * DB, "ring schedule is written for 64-row key tiles");
 
   __shared__ __attribute__((aligned(1024))) short smem[L::TOTAL_ELEMS];
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
   const int c = lane & 31, h = lane >> 5;
   const int i16 = lane & 15, g2 = (lane >> 4) & 1;
 
@@ -385,20 +331,23 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
 
   const int kv_end = min(q0 + kFwdBlockQ, p.seqlen_k);
   const int n_tiles = (kv_end + BKV - 1) / BKV;
+  // Tiles this wave multiplies: those starting at or before its last query row.
+  const int n_mine = min(n_tiles, (q0w + 31) / BKV + 1);
+  // Leading tiles that need no mask (entirely at or below the wave's first row, inside the keys).
   const int n_full = max(0, min(min(q0w + 1, p.seqlen_k) / BKV, n_tiles));
   const int n_inside = p.seqlen_k / BKV;  // tiles whose every row exists
 
-  auto issue_tile = [&](int t) {
-    short *stage = smem + (t & 1) * L::STAGE_ELEMS;
-    if (t < n_inside) {
-      kload.issue(t * BKV, stage);
-      vload.issue(t * BKV, stage + L::TILE_ELEMS);
-    } else {
-      kload.issue_clamped(t * BKV, p.seqlen_k, stage);
-      vload.issue_clamped(t * BKV, p.seqlen_k, stage + L::TILE_ELEMS);
-    }
+  auto issue_k = [&](int t, int stage) {
+    short *dst = smem + L::K_BASE + stage * L::TILE_ELEMS;
+    if (t < n_inside) kload.issue(t * BKV, dst); else kload.issue_clamped(t * BKV, p.seqlen_k, dst);
   };
-  issue_tile(0);
+  auto issue_v = [&](int t, int stage) {
+    short *dst = smem + L::V_BASE + stage * L::TILE_ELEMS;
+    if (t < n_inside) vload.issue(t * BKV, dst); else vload.issue_clamped(t * BKV, p.seqlen_k, dst);
+  };
+  issue_k(0, 0);
+  issue_v(0, 0);
+  if (n_tiles > 1) issue_k(1, 1);
 
   // Q^T fragments (B operand of S^T = K Q^T): lane (c, h) holds Q[q0w + c][16 ks + 8 h + j].
   s16x8 qf[KS];
@@ -410,18 +359,20 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
     for (int ks = 0; ks < KS; ks++) qf[ks] = load_chunk(rp, 16 * ks + 8 * h, DP, ok, true);
   }
 
-  // Fragment offsets inside a tile (swizzled); tile-relative row blocks are added as immediates.
-  int kaddr[KS], valo[DB], vahi[DB];
+  // Fragment addresses inside a tile (swizzled).  Stage and row-block offsets are compile-time
+  // constants that end up in the instructions' immediate offset fields.
+  const short *kptr[KS];
+  const short *vlo[DB], *vhi[DB];
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) kaddr[ks] = swz_off<DP>(c, 2 * ks + h);
+  for (int ks = 0; ks < KS; ks++) kptr[ks] = smem + L::K_BASE + swz_off<DP>(c, 2 * ks + h);
   {
     const int rowlo = 4 * h + (i16 >> 2);
     const int sub = (i16 & 1) * 4;
 #pragma unroll
     for (int db = 0; db < DB; db++) {
       const int chunk = 4 * db + 2 * g2 + ((i16 & 3) >> 1);
-      valo[db] = swz_off<DP>(rowlo, chunk) + sub;
-      vahi[db] = swz_off<DP>(rowlo + 8, chunk) + sub;
+      vlo[db] = smem + L::V_BASE + swz_off<DP>(rowlo, chunk) + sub;
+      vhi[db] = smem + L::V_BASE + swz_off<DP>(rowlo + 8, chunk) + sub;
     }
   }
 
@@ -430,37 +381,174 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   for (int db = 0; db < DB; db++)
 #pragma unroll
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
-  float m_ref = -INFINITY;
+  float m_ref = -INFINITY;  // maximum (raw scores) the probabilities are formed against
   float l_run = 0.f;
   const int qrow = q0w + c;
 
   wait_vmem_all();
   __syncthreads();
 
-  for (int t = 0; t < n_tiles; t++) {
-    const int kvt = t * BKV;
-    if (t + 1 < n_tiles) issue_tile(t + 1);
+#ifdef FA2_PHASE_TIMING
+  long long phase_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  long long tick_ = __builtin_amdgcn_s_memtime();
+  const long long core0_ = tick_, wall0_ = wall_clock64();
+#endif
+  // Ring of operand fragments, preloaded with K tile 0, block 0.
+  s16x8 ring[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) ring[ks] = *reinterpret_cast<const s16x8 *>(kptr[ks]);
 
-    const short *sk = smem + (t & 1) * L::STAGE_ELEMS;
-    const short *sv = sk + L::TILE_ELEMS;
-    if (t < n_full) {
-      fwd_tile_direct<T, DP, BKV, false>(sk, sv, qf, oacc, m_ref, l_run, p.scale_log2, kvt, qrow,
-                                         p.seqlen_k, kaddr, valo, vahi);
-    } else if (kvt <= q0w + 31) {
-      fwd_tile_direct<T, DP, BKV, true>(sk, sv, qf, oacc, m_ref, l_run, p.scale_log2, kvt, qrow,
-                                        p.seqlen_k, kaddr, valo, vahi);
+  // One key tile; STAGE (= t & 1) is a template argument so that every LDS address is a
+  // register plus an immediate.
+  auto tile = [&](int t, auto stage_tag) {
+    constexpr int STAGE = decltype(stage_tag)::value;
+    constexpr int KOFF = STAGE * L::TILE_ELEMS;         // K_t and V_t live in stage t & 1
+    constexpr int KOFF_NEXT = (1 - STAGE) * L::TILE_ELEMS;
+    const int kvt = t * BKV;
+    const bool mine = t < n_mine;
+
+    // ---- S^T = K Q^T -----------------------------------------------------------------------
+    FA2_TICK(4);
+    f32x16 s[MB];
+    if (mine) {
+      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      s[0] = zero;
+      s[1] = zero;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        s[0] = Elem<T>::mfma(ring[ks], qf[ks], s[0]);
+        ring[ks] = *reinterpret_cast<const s16x8 *>(kptr[ks] + KOFF + 32 * DP);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) s[1] = Elem<T>::mfma(ring[ks], qf[ks], s[1]);
     }
 
+    // Everyone is done with K_t and V_{t-1}; K_{t+1} and V_t have landed.
+    FA2_TICK(0);
     wait_vmem_all();
+    FA2_TICK(5);
     __syncthreads();
+    FA2_TICK(1);
+    if (t + 2 < n_tiles) issue_k(t + 2, STAGE);
+    if (t + 1 < n_tiles) issue_v(t + 1, 1 - STAGE);
+
+    if (mine) {
+      // V^T fragments for the first two k-steps, ahead of the softmax arithmetic.
+#pragma unroll
+      for (int ks2 = 0; ks2 < 2; ks2++)
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+          s16x4 lo = lds_read_tr(vlo[db] + KOFF + 16 * ks2 * DP);
+          s16x4 hi = lds_read_tr(vhi[db] + KOFF + 16 * ks2 * DP);
+          ring[ks2 * DB + db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+
+      // ---- online softmax ------------------------------------------------------------------
+      if (t >= n_full) {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            const int kv = kvt + 32 * mb + 8 * (i >> 2) + 4 * h + (i & 3);
+            if (kv > qrow || kv >= p.seqlen_k) s[mb][i] = -INFINITY;
+          }
+      }
+      float mloc = s[0][0];
+#pragma unroll
+      for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) mloc = fmaxf(mloc, s[mb][i]);
+      mloc = max_over_halves(mloc);
+
+      // Raise the reference maximum only when some row needs it (wave-uniform branch; always
+      // taken on the first tile, where m_ref is -inf).
+      const bool grow = (mloc - m_ref) * p.scale_log2 > kRescaleSlack;
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+        const float m_new = fmaxf(m_ref, mloc);
+        const float alpha = fast_exp2((m_ref - m_new) * p.scale_log2);
+        m_ref = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+      }
+      const float mc = m_ref * p.scale_log2;
+
+      s16x8 pf[KS2];
+#pragma unroll
+      for (int mb = 0; mb < MB; mb++) {
+        f32x16 e;
+#pragma unroll
+        for (int i = 0; i < 16; i++) e[i] = fast_exp2(s[mb][i] * p.scale_log2 - mc);
+        f32x8 lo = {e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]};
+        f32x8 hi = {e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]};
+        pf[2 * mb] = Elem<T>::pack8(lo);
+        pf[2 * mb + 1] = Elem<T>::pack8(hi);
+      }
+      // Row sums from the rounded probabilities, two per instruction.
+#pragma unroll
+      for (int ks2 = 0; ks2 < KS2; ks2++) {
+        typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 w = __builtin_bit_cast(u32x4, pf[ks2]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) l_run = Elem<T>::add_pair(w[j], l_run);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      FA2_TICK(2);
+
+      // ---- O^T += V^T P^T; the ring refills with later V fragments, then with K_{t+1} -------
+      const bool next_mine = (t + 1) < n_mine;
+#pragma unroll
+      for (int ks2 = 0; ks2 < KS2; ks2++) {
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+          const int slot = (ks2 & 1) * DB + db;
+          oacc[db] = Elem<T>::mfma(ring[slot], pf[ks2], oacc[db]);
+          if (ks2 + 2 < KS2) {
+            s16x4 lo = lds_read_tr(vlo[db] + KOFF + 16 * (ks2 + 2) * DP);
+            s16x4 hi = lds_read_tr(vhi[db] + KOFF + 16 * (ks2 + 2) * DP);
+            ring[slot] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          } else if (next_mine) {
+            ring[slot] = *reinterpret_cast<const s16x8 *>(kptr[(ks2 - (KS2 - 2)) * DB + db] + KOFF_NEXT);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      FA2_TICK(3);
+    }
+  };
+
+  for (int t = 0; t < n_tiles; t += 2) {
+    tile(t, std::integral_constant<int, 0>{});
+    if (t + 1 < n_tiles) tile(t + 1, std::integral_constant<int, 1>{});
   }
 
+#ifdef FA2_PHASE_TIMING
+  phase_acc[6] = __builtin_amdgcn_s_memtime() - core0_;
+  phase_acc[7] = wall_clock64() - wall0_;
+  if (blockIdx.x == FA2_PHASE_TIMING && lane == 0)
+    for (int i = 0; i < 8; i++) fa2_phase_cycles[wave][i] = phase_acc[i];
+  if (tid == 0 && blockIdx.x < 8192) {
+    unsigned hwid, xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    fa2_wg_times[blockIdx.x][0] = wall0_;
+    fa2_wg_times[blockIdx.x][1] = wall_clock64();
+    fa2_wg_times[blockIdx.x][2] = hwid;
+    fa2_wg_times[blockIdx.x][3] = xcc;
+  }
+#endif
   const float l_tot = sum_over_halves(l_run);
   const float inv_l = 1.f / l_tot;
   if (h == 0 && q0w + c < p.seqlen_q) LSE[q0w + c] = m_ref * p.scale + __logf(l_tot);
   if (qt == p.n_qtiles - 1) {
     for (int r = p.seqlen_q + tid; r < p.seqlen_q_rounded; r += NTHREADS) LSE[r] = 0.f;
   }
+  // The patch overlays the stages: wait until every wave has finished its last tile.
+  __syncthreads();
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(oacc, inv_l, patch, O + (int64_t)q0w * p.o.stride_seq,
                               p.o.stride_seq, p.seqlen_q - q0w, DP, true);
