@@ -359,13 +359,10 @@ int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const 
   return FA2_OK;
 }
 
-#ifdef FA2_PHASE_TIMING
-// Debug build only (never declared in the public header): copies the phase counters to the host.
-int fa2_debug_phase_cycles(long long *out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(fa2::fa2_phase_cycles), sizeof(long long) * 64);
-}
-int fa2_debug_wg_times(long long *out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(fa2::fa2_wg_times), sizeof(long long) * 8192 * 4);
+#ifdef FA2_WG_STAMPS
+// Debug build only (never declared in the public header): copies the workgroup stamps to the host.
+int fa2_debug_wg_stamps(long long *out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(fa2::fa2_wg_stamps), sizeof(long long) * 8192 * 4);
 }
 #endif
 

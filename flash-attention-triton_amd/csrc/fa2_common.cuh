@@ -53,6 +53,12 @@ struct Elem<__bf16> {
   static __device__ __forceinline__ s16x4 pack4(f32x4 x) {
     return __builtin_bit_cast(s16x4, __builtin_convertvector(x, bf16x4));
   }
+  static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const f32x2 x = {lo, hi};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(x, bf16x2));
+  }
   static __device__ __forceinline__ float to_float(short x) {
     return __builtin_bit_cast(float, ((unsigned)(unsigned short)x) << 16);
   }
@@ -76,6 +82,12 @@ struct Elem<_Float16> {
   static __device__ __forceinline__ s16x4 pack4(f32x4 x) {
     return __builtin_bit_cast(s16x4, __builtin_convertvector(x, f16x4));
   }
+  static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const f32x2 x = {lo, hi};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(x, f16x2));
+  }
   static __device__ __forceinline__ float to_float(short x) {
     return (float)__builtin_bit_cast(_Float16, x);
   }
@@ -86,8 +98,20 @@ struct Elem<_Float16> {
   }
 };
 
+// 32-bit pointer into LDS.
+typedef const __attribute__((address_space(3))) short *lds_cptr;
+__device__ __forceinline__ lds_cptr to_lds(const short *p) {
+  return (lds_cptr)(const __attribute__((address_space(3))) void *)p;
+}
+__device__ __forceinline__ s16x8 lds_read_128(lds_cptr p) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) s16x8 *>(p);
+}
+
 // Transposing 64-bit LDS read (ds_read_b64_tr_b16).
 __device__ __forceinline__ s16x4 lds_read_tr(const short *p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p));
+}
+__device__ __forceinline__ s16x4 lds_read_tr(lds_cptr p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p));
 }
 
@@ -221,8 +245,8 @@ __device__ __forceinline__ int swz_off(int r, int c) { return r * DP + ((c ^ swz
 // serialise the prefetch.  The callers order these loads against LDS reads themselves with
 // `s_waitcnt vmcnt(0)` followed by a workgroup barrier.
 __device__ __forceinline__ void load_lds_16(const short *gsrc, short *lds_wave_base) {
-  const unsigned lds_addr =
-      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base;
+  const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
+      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base);
   asm volatile(
       "s_mov_b32 m0, %1\n\t"
       "s_nop 0\n\t"
@@ -234,8 +258,15 @@ __device__ __forceinline__ void load_lds_16(const short *gsrc, short *lds_wave_b
 // Same with the address split into a wave-uniform base (SGPR pair) and a per-lane byte offset.
 __device__ __forceinline__ void load_lds_16(const short *uniform_base, unsigned lane_byte_offset,
                                             short *lds_wave_base) {
-  const unsigned lds_addr =
-      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base;
+  const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
+      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base);
+  // State the uniformity the "s" constraints need (folds away when the value is already scalar).
+  const uint64_t raw = (uint64_t)(uintptr_t)uniform_base;
+  // (readfirstlane returns a signed int: go through unsigned so the low word is not sign-extended)
+  const uint64_t hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(raw >> 32));
+  const uint64_t lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)raw);
+  const uint64_t ubase = (hi << 32) | lo;
+  uniform_base = (const short *)(uintptr_t)ubase;
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
       "s_nop 0\n\t"

@@ -263,50 +263,56 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams 
 // ------------------------------------------------------------------------------------------
 // Fast path: head dimension equal to the padded one and 16-byte aligned rows.
 //
-//  * K and V tiles go straight from global memory into swizzled, unpadded LDS
-//    (global_load_lds_dwordx4: no staging registers, no LDS stores), two stages each.
-//  * One workgroup barrier per tile, placed between the two GEMMs.  At that point every wave has
-//    finished reading K_t and V_{t-1}, so K_{t+2} and V_{t+1} are issued right after it and have
-//    a whole tile of time to land.
-//  * MFMA operand fragments travel through a ring of DP/16 registers-sets that is always loaded
-//    ahead of use: while S^T block 0 is multiplied the ring refills with block 1; V^T fragments
-//    are fetched before the softmax arithmetic starts; the tail of the P V GEMM refills the ring
-//    with the next tile's first K fragments.  LDS latency is therefore never waited for.
+//  * K and V tiles (64 rows) go straight from global memory into swizzled, unpadded LDS
+//    (global_load_lds_dwordx4: no staging registers, no LDS stores); three K stages and two V
+//    stages, one workgroup barrier per tile.
+//  * The work is software-pipelined over 32-key blocks so that every MFMA has independent
+//    vector work of the same wave next to it (about four VALU instructions issue for free under
+//    a 32x32x16 MFMA, and short alternating phases are also what lets two waves of one SIMD
+//    overlap).  For block j:
+//        X(j): S_{j+1}^T = K_{j+1} Q^T   interleaved with   P_j = exp2(scale*S_j - m), row sums
+//        Y(j): O^T += V_j^T P_j^T         interleaved with   row maximum of S_{j+1}
+//    The two score buffers alternate roles, so pipelining costs no extra registers.
+//  * MFMA operand fragments travel through a ring of DP/16 register sets that is refilled as it
+//    is consumed (K fragments of block j+2 during Y(j), V fragments of block j during X(j)), so
+//    LDS latency hides behind the MFMAs.
 // ------------------------------------------------------------------------------------------
 template <int DP, int BKV>
 struct FwdDirectLayout {
   static constexpr int TILE_ELEMS = BKV * DP;
-  static constexpr int K_BASE = 0;                 // two K stages
-  static constexpr int V_BASE = 2 * TILE_ELEMS;    // two V stages
+  static constexpr int K_STAGES = 3, V_STAGES = 2;
+  static constexpr int K_BASE = 0;
+  static constexpr int V_BASE = K_STAGES * TILE_ELEMS;
+  static constexpr int STAGE_ELEMS = (K_STAGES + V_STAGES) * TILE_ELEMS;
   static constexpr int PATCH_ELEMS = kFwdWaves * 32 * (DP + 8);
-  static constexpr int TOTAL_ELEMS = (4 * TILE_ELEMS > PATCH_ELEMS) ? 4 * TILE_ELEMS : PATCH_ELEMS;
+  static constexpr int TOTAL_ELEMS = (STAGE_ELEMS > PATCH_ELEMS) ? STAGE_ELEMS : PATCH_ELEMS;
 };
 
 // s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt fields left at their maxima).
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-#ifdef FA2_PHASE_TIMING
-// Debug build only: cycles spent in each phase, summed over tiles, for workgroup 0's waves.
-__device__ long long fa2_phase_cycles[8][8];
-__device__ long long fa2_wg_times[8192][4];
-#define FA2_TICK(slot)                                        \
-  do {                                                        \
-    const long long now_ = __builtin_amdgcn_s_memtime();      \
-    if (blockIdx.x == FA2_PHASE_TIMING) phase_acc[slot] += now_ - tick_; \
-    tick_ = now_;                                             \
-  } while (0)
+// Scheduling-group masks of __builtin_amdgcn_sched_group_barrier.
+constexpr int kSgValu = 0x002, kSgMfma = 0x008, kSgDsRead = 0x100, kSgTrans = 0x400;
+
+#ifdef FA2_WG_STAMPS
+// Debug build only: wall-clock (100 MHz) stamps per workgroup: start, loop start, loop end, end.
+__device__ long long fa2_wg_stamps[8192][4];
+#define FA2_STAMP(slot) do { if (threadIdx.x == 0 && blockIdx.x < 8192) fa2_wg_stamps[blockIdx.x][slot] = wall_clock64(); } while (0)
 #else
-#define FA2_TICK(slot) do {} while (0)
+#define FA2_STAMP(slot) do {} while (0)
 #endif
 
 template <typename T, int DP, int BKV>
 __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const FwdParams p) {
   using L = FwdDirectLayout<DP, BKV>;
-  constexpr int KS = DP / 16, DB = DP / 32, MB = BKV / 32, KS2 = BKV / 16;
+  constexpr int KS = DP / 16, DB = DP / 32;
   constexpr int NTHREADS = 64 * kFwdWaves;
-  static_assert(MB == 2 && KS2 == 4 && KS == 2 * DB, "ring schedule is written for 64-row key tiles");
+  constexpr int BLK = 32;  // keys per pipeline block
+  static_assert(BKV == 2 * BLK && KS == 2 * DB, "schedule is written for 64-row tiles of two blocks");
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
   __shared__ __attribute__((aligned(1024))) short smem[L::TOTAL_ELEMS];
+  FA2_STAMP(0);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -328,26 +334,29 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   float *LSE = p.lse + (int64_t)bh * p.seqlen_q_rounded;
 
   const TileLoader<DP, BKV, kFwdWaves> kload(K, p.k.stride_seq), vload(V, p.v.stride_seq);
+  const int seqlen_k = p.seqlen_k;
+  const float scale_log2 = p.scale_log2;
 
-  const int kv_end = min(q0 + kFwdBlockQ, p.seqlen_k);
+  const int kv_end = min(q0 + kFwdBlockQ, seqlen_k);
   const int n_tiles = (kv_end + BKV - 1) / BKV;
-  // Tiles this wave multiplies: those starting at or before its last query row.
-  const int n_mine = min(n_tiles, (q0w + 31) / BKV + 1);
-  // Leading tiles that need no mask (entirely at or below the wave's first row, inside the keys).
-  const int n_full = max(0, min(min(q0w + 1, p.seqlen_k) / BKV, n_tiles));
-  const int n_inside = p.seqlen_k / BKV;  // tiles whose every row exists
+  // Blocks this wave multiplies: those that exist and start at or before its last query row.
+  const int n_mine = min((kv_end + BLK - 1) / BLK, q0w / BLK + 1);
+  // Leading blocks that need no mask (entirely at or below the wave's first row, inside the keys).
+  const int n_full = min(q0w + 1, seqlen_k) / BLK;
+  const int n_inside = seqlen_k / BKV;  // tiles whose every row exists
 
-  auto issue_k = [&](int t, int stage) {
-    short *dst = smem + L::K_BASE + stage * L::TILE_ELEMS;
-    if (t < n_inside) kload.issue(t * BKV, dst); else kload.issue_clamped(t * BKV, p.seqlen_k, dst);
+  auto issue_k = [&](int t) {
+    short *dst = smem + L::K_BASE + (t % L::K_STAGES) * L::TILE_ELEMS;
+    if (t < n_inside) kload.issue(t * BKV, dst); else kload.issue_clamped(t * BKV, seqlen_k, dst);
   };
-  auto issue_v = [&](int t, int stage) {
-    short *dst = smem + L::V_BASE + stage * L::TILE_ELEMS;
-    if (t < n_inside) vload.issue(t * BKV, dst); else vload.issue_clamped(t * BKV, p.seqlen_k, dst);
+  auto issue_v = [&](int t) {
+    short *dst = smem + L::V_BASE + (t % L::V_STAGES) * L::TILE_ELEMS;
+    if (t < n_inside) vload.issue(t * BKV, dst); else vload.issue_clamped(t * BKV, seqlen_k, dst);
   };
-  issue_k(0, 0);
-  issue_v(0, 0);
-  if (n_tiles > 1) issue_k(1, 1);
+  issue_k(0);
+  issue_v(0);
+  if (n_tiles > 1) { issue_k(1); issue_v(1); }
+  if (n_tiles > 2) issue_k(2);
 
   // Q^T fragments (B operand of S^T = K Q^T): lane (c, h) holds Q[q0w + c][16 ks + 8 h + j].
   s16x8 qf[KS];
@@ -359,22 +368,31 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
     for (int ks = 0; ks < KS; ks++) qf[ks] = load_chunk(rp, 16 * ks + 8 * h, DP, ok, true);
   }
 
-  // Fragment addresses inside a tile (swizzled).  Stage and row-block offsets are compile-time
-  // constants that end up in the instructions' immediate offset fields.
-  const short *kptr[KS];
-  const short *vlo[DB], *vhi[DB];
+  // Fragment addresses (swizzled, 32-bit LDS pointers).  kcur points into the stage of the K tile
+  // after the current one, vcur into the stage of the current V tile; both advance by a uniform
+  // amount per tile, and half-tile offsets are immediates.
+  lds_cptr kcur[KS], vlo[DB], vhi[DB];
+  const lds_cptr lds0 = to_lds(smem);
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) kptr[ks] = smem + L::K_BASE + swz_off<DP>(c, 2 * ks + h);
+  for (int ks = 0; ks < KS; ks++) kcur[ks] = lds0 + L::K_BASE + swz_off<DP>(c, 2 * ks + h);
   {
     const int rowlo = 4 * h + (i16 >> 2);
     const int sub = (i16 & 1) * 4;
 #pragma unroll
     for (int db = 0; db < DB; db++) {
       const int chunk = 4 * db + 2 * g2 + ((i16 & 3) >> 1);
-      vlo[db] = smem + L::V_BASE + swz_off<DP>(rowlo, chunk) + sub;
-      vhi[db] = smem + L::V_BASE + swz_off<DP>(rowlo + 8, chunk) + sub;
+      vlo[db] = lds0 + L::V_BASE + swz_off<DP>(rowlo, chunk) + sub;
+      vhi[db] = lds0 + L::V_BASE + swz_off<DP>(rowlo + 8, chunk) + sub;
     }
   }
+  // K fragment ks of the half-tile `half` of the tile kcur points at.
+  auto k_frag = [&](int half, int ks) { return lds_read_128(kcur[ks] + half * BLK * DP); };
+  // V^T fragment (k-step ks2 in {0,1} of half-tile `half`, head-dim block db) of the tile vcur points at.
+  auto v_frag = [&](int half, int ks2, int db) -> s16x8 {
+    s16x4 lo = lds_read_tr(vlo[db] + half * BLK * DP + 16 * ks2 * DP);
+    s16x4 hi = lds_read_tr(vhi[db] + half * BLK * DP + 16 * ks2 * DP);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
 
   f32x16 oacc[DB];
 #pragma unroll
@@ -382,176 +400,166 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
 #pragma unroll
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
   float m_ref = -INFINITY;  // maximum (raw scores) the probabilities are formed against
-  float l_run = 0.f;
+  float l_run = 0.f;        // this lane's share of the running sum (its half of the key rows)
   const int qrow = q0w + c;
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  auto apply_mask = [&](f32x16 &s, int kv0) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int kv = kv0 + 8 * (i >> 2) + 4 * h + (i & 3);
+      if (kv > qrow || kv >= seqlen_k) s[i] = -INFINITY;
+    }
+  };
+  auto row_max = [&](const f32x16 &s) {
+    float m = s[0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) m = fmaxf(m, s[i]);
+    return max_over_halves(m);
+  };
+  // P = exp2(scale*S - scale*m) rounded to T, plus the row sums of the rounded values.
+  auto softmax_block = [&](const f32x16 &s, s16x8 (&pf)[2]) {
+    const float mc = m_ref * scale_log2;
+    f32x16 e;
+#pragma unroll
+    for (int i = 0; i < 16; i++) e[i] = fast_exp2(s[i] * scale_log2 - mc);
+    f32x8 lo = {e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]};
+    f32x8 hi = {e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]};
+    pf[0] = Elem<T>::pack8(lo);
+    pf[1] = Elem<T>::pack8(hi);
+#pragma unroll
+    for (int ks2 = 0; ks2 < 2; ks2++) {
+      const u32x4 w = __builtin_bit_cast(u32x4, pf[ks2]);
+#pragma unroll
+      for (int j = 0; j < 4; j++) l_run = Elem<T>::add_pair(w[j], l_run);
+    }
+  };
+  // Raise the reference maximum when some row overshoots it by more than the slack.
+  auto maybe_rescale = [&](float mloc) {
+    const bool grow = (mloc - m_ref) * scale_log2 > kRescaleSlack;
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float m_new = fmaxf(m_ref, mloc);
+      const float alpha = fast_exp2((m_ref - m_new) * scale_log2);
+      m_ref = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+    }
+  };
 
   wait_vmem_all();
   __syncthreads();
 
-#ifdef FA2_PHASE_TIMING
-  long long phase_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  long long tick_ = __builtin_amdgcn_s_memtime();
-  const long long core0_ = tick_, wall0_ = wall_clock64();
-#endif
-  // Ring of operand fragments, preloaded with K tile 0, block 0.
+  // ---- prologue: S_0, its row maximum, ring <- K fragments of block 1 -------------------------
   s16x8 ring[KS];
+  f32x16 sa, sb;
+  {
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) ring[ks] = *reinterpret_cast<const s16x8 *>(kptr[ks]);
-
-  // One key tile; STAGE (= t & 1) is a template argument so that every LDS address is a
-  // register plus an immediate.
-  auto tile = [&](int t, auto stage_tag) {
-    constexpr int STAGE = decltype(stage_tag)::value;
-    constexpr int KOFF = STAGE * L::TILE_ELEMS;         // K_t and V_t live in stage t & 1
-    constexpr int KOFF_NEXT = (1 - STAGE) * L::TILE_ELEMS;
-    const int kvt = t * BKV;
-    const bool mine = t < n_mine;
-
-    // ---- S^T = K Q^T -----------------------------------------------------------------------
-    FA2_TICK(4);
-    f32x16 s[MB];
-    if (mine) {
-      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      s[0] = zero;
-      s[1] = zero;
+    for (int ks = 0; ks < KS; ks++) ring[ks] = k_frag(0, ks);
+    sa = zero;
 #pragma unroll
-      for (int ks = 0; ks < KS; ks++) {
-        s[0] = Elem<T>::mfma(ring[ks], qf[ks], s[0]);
-        ring[ks] = *reinterpret_cast<const s16x8 *>(kptr[ks] + KOFF + 32 * DP);
+    for (int ks = 0; ks < KS; ks++) sa = Elem<T>::mfma(ring[ks], qf[ks], sa);
+    if (0 >= n_full) apply_mask(sa, 0);
+    m_ref = row_max(sa);  // finite: every query row sees key 0
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) ring[ks] = k_frag(1, ks);
+    // From here on kcur addresses K tile 1 (the tile after the current one).
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) kcur[ks] += L::TILE_ELEMS;
+  }
+
+  // One block step: scur holds S_j (maximum already accounted for), snxt receives S_{j+1}.
+  // HALF (= j & 1) selects the half-tile: V_j is half HALF of the current V tile and K_{j+2} is
+  // half HALF of the next K tile.
+  //
+  // The step is hand-interleaved: each unit is one MFMA, the LDS reads that refill the ring slot
+  // it just freed, and a few vector instructions; a scheduling fence after every unit keeps the
+  // compiler from regrouping them (which would lengthen live ranges past the register file).
+  // S_{j+1} and the K fragments of block j+2 are produced even when those blocks are not this
+  // wave's (the values are then never used), so that there is a single code path.
+  auto step = [&](int j, auto half_tag, f32x16 &scur, f32x16 &snxt) {
+    constexpr int HALF = decltype(half_tag)::value;
+    if (j >= n_mine) return;
+    const float mc = m_ref * scale_log2;
+    typedef unsigned u32x4v __attribute__((ext_vector_type(4)));
+    u32x4v w[2];  // packed probabilities, two per word: w[0] = k-step 0, w[1] = k-step 1
+    snxt = zero;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      snxt = Elem<T>::mfma(ring[ks], qf[ks], snxt);
+      ring[ks] = v_frag(HALF, ks / DB, ks % DB);
+#pragma unroll
+      for (int u = 0; u < 8 / KS; u++) {
+        const int i = (8 / KS) * ks + u;  // probability pair (2i, 2i+1) of the 32 in the block
+        const float e0 = fast_exp2(scur[2 * i] * scale_log2 - mc);
+        const float e1 = fast_exp2(scur[2 * i + 1] * scale_log2 - mc);
+        w[i / 4][i % 4] = Elem<T>::pack2(e0, e1);
+        l_run += e0;
+        l_run += e1;
+      }
+      // Pin the arithmetic to this unit: without a use here the optimiser sinks it past the
+      // branch below, next to the MFMAs that consume it.
+      asm volatile("" : "+v"(l_run));
+      if (ks == KS / 2 - 1) asm volatile("" : "+v"(w[0]));
+      if (ks == KS - 1) asm volatile("" : "+v"(w[1]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (j + 1 >= n_full) apply_mask(snxt, (j + 1) * BLK);
+    const s16x8 pf[2] = {__builtin_bit_cast(s16x8, w[0]), __builtin_bit_cast(s16x8, w[1])};
+    float mloc = fmaxf(snxt[0], snxt[1]);
+#pragma unroll
+    for (int ks2 = 0; ks2 < 2; ks2++) {
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const int slot = ks2 * DB + db;
+        oacc[db] = Elem<T>::mfma(ring[slot], pf[ks2], oacc[db]);
+        ring[slot] = k_frag(HALF, slot);
+        if (slot >= 1 && 2 * slot + 1 < 16) mloc = fmaxf(fmaxf(mloc, snxt[2 * slot]), snxt[2 * slot + 1]);
+        asm volatile("" : "+v"(mloc));
         __builtin_amdgcn_sched_barrier(0);
       }
-#pragma unroll
-      for (int ks = 0; ks < KS; ks++) s[1] = Elem<T>::mfma(ring[ks], qf[ks], s[1]);
     }
-
-    // Everyone is done with K_t and V_{t-1}; K_{t+1} and V_t have landed.
-    FA2_TICK(0);
-    wait_vmem_all();
-    FA2_TICK(5);
-    __syncthreads();
-    FA2_TICK(1);
-    if (t + 2 < n_tiles) issue_k(t + 2, STAGE);
-    if (t + 1 < n_tiles) issue_v(t + 1, 1 - STAGE);
-
-    if (mine) {
-      // V^T fragments for the first two k-steps, ahead of the softmax arithmetic.
 #pragma unroll
-      for (int ks2 = 0; ks2 < 2; ks2++)
-#pragma unroll
-        for (int db = 0; db < DB; db++) {
-          s16x4 lo = lds_read_tr(vlo[db] + KOFF + 16 * ks2 * DP);
-          s16x4 hi = lds_read_tr(vhi[db] + KOFF + 16 * ks2 * DP);
-          ring[ks2 * DB + db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-      __builtin_amdgcn_sched_barrier(0);
-
-      // ---- online softmax ------------------------------------------------------------------
-      if (t >= n_full) {
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const int kv = kvt + 32 * mb + 8 * (i >> 2) + 4 * h + (i & 3);
-            if (kv > qrow || kv >= p.seqlen_k) s[mb][i] = -INFINITY;
-          }
-      }
-      float mloc = s[0][0];
-#pragma unroll
-      for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) mloc = fmaxf(mloc, s[mb][i]);
-      mloc = max_over_halves(mloc);
-
-      // Raise the reference maximum only when some row needs it (wave-uniform branch; always
-      // taken on the first tile, where m_ref is -inf).
-      const bool grow = (mloc - m_ref) * p.scale_log2 > kRescaleSlack;
-      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-        const float m_new = fmaxf(m_ref, mloc);
-        const float alpha = fast_exp2((m_ref - m_new) * p.scale_log2);
-        m_ref = m_new;
-        l_run *= alpha;
-#pragma unroll
-        for (int db = 0; db < DB; db++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
-      }
-      const float mc = m_ref * p.scale_log2;
-
-      s16x8 pf[KS2];
-#pragma unroll
-      for (int mb = 0; mb < MB; mb++) {
-        f32x16 e;
-#pragma unroll
-        for (int i = 0; i < 16; i++) e[i] = fast_exp2(s[mb][i] * p.scale_log2 - mc);
-        f32x8 lo = {e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]};
-        f32x8 hi = {e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]};
-        pf[2 * mb] = Elem<T>::pack8(lo);
-        pf[2 * mb + 1] = Elem<T>::pack8(hi);
-      }
-      // Row sums from the rounded probabilities, two per instruction.
-#pragma unroll
-      for (int ks2 = 0; ks2 < KS2; ks2++) {
-        typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-        const u32x4 w = __builtin_bit_cast(u32x4, pf[ks2]);
-#pragma unroll
-        for (int j = 0; j < 4; j++) l_run = Elem<T>::add_pair(w[j], l_run);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      FA2_TICK(2);
-
-      // ---- O^T += V^T P^T; the ring refills with later V fragments, then with K_{t+1} -------
-      const bool next_mine = (t + 1) < n_mine;
-#pragma unroll
-      for (int ks2 = 0; ks2 < KS2; ks2++) {
-#pragma unroll
-        for (int db = 0; db < DB; db++) {
-          const int slot = (ks2 & 1) * DB + db;
-          oacc[db] = Elem<T>::mfma(ring[slot], pf[ks2], oacc[db]);
-          if (ks2 + 2 < KS2) {
-            s16x4 lo = lds_read_tr(vlo[db] + KOFF + 16 * (ks2 + 2) * DP);
-            s16x4 hi = lds_read_tr(vhi[db] + KOFF + 16 * (ks2 + 2) * DP);
-            ring[slot] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          } else if (next_mine) {
-            ring[slot] = *reinterpret_cast<const s16x8 *>(kptr[(ks2 - (KS2 - 2)) * DB + db] + KOFF_NEXT);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      FA2_TICK(3);
-    }
+    for (int i = 2 * KS; i < 16; i++) mloc = fmaxf(mloc, snxt[i]);
+    mloc = max_over_halves(mloc);
+    if (j + 1 < n_mine) maybe_rescale(mloc);
   };
 
-  for (int t = 0; t < n_tiles; t += 2) {
-    tile(t, std::integral_constant<int, 0>{});
-    if (t + 1 < n_tiles) tile(t + 1, std::integral_constant<int, 1>{});
+  FA2_STAMP(1);
+  for (int t = 0; t < n_tiles; t++) {
+    step(2 * t, std::integral_constant<int, 0>{}, sa, sb);
+    step(2 * t + 1, std::integral_constant<int, 1>{}, sb, sa);
+    // Every wave is done with K_t and V_t; K_{t+2} and V_{t+1} (issued one tile ago) have landed.
+    wait_vmem_all();
+    __syncthreads();
+    if (t + 3 < n_tiles) issue_k(t + 3);
+    if (t + 2 < n_tiles) issue_v(t + 2);
+    // Advance the fragment pointers to K tile t+2 and V tile t+1 (stages are used round-robin).
+    const int dk = ((t + 2) % L::K_STAGES == 0) ? -(L::K_STAGES - 1) * L::TILE_ELEMS : L::TILE_ELEMS;
+    const int dv = ((t + 1) % L::V_STAGES == 0) ? -(L::V_STAGES - 1) * L::TILE_ELEMS : L::TILE_ELEMS;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) kcur[ks] += dk;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      vlo[db] += dv;
+      vhi[db] += dv;
+    }
   }
 
-#ifdef FA2_PHASE_TIMING
-  phase_acc[6] = __builtin_amdgcn_s_memtime() - core0_;
-  phase_acc[7] = wall_clock64() - wall0_;
-  if (blockIdx.x == FA2_PHASE_TIMING && lane == 0)
-    for (int i = 0; i < 8; i++) fa2_phase_cycles[wave][i] = phase_acc[i];
-  if (tid == 0 && blockIdx.x < 8192) {
-    unsigned hwid, xcc;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-    fa2_wg_times[blockIdx.x][0] = wall0_;
-    fa2_wg_times[blockIdx.x][1] = wall_clock64();
-    fa2_wg_times[blockIdx.x][2] = hwid;
-    fa2_wg_times[blockIdx.x][3] = xcc;
-  }
-#endif
+  FA2_STAMP(2);
   const float l_tot = sum_over_halves(l_run);
   const float inv_l = 1.f / l_tot;
   if (h == 0 && q0w + c < p.seqlen_q) LSE[q0w + c] = m_ref * p.scale + __logf(l_tot);
   if (qt == p.n_qtiles - 1) {
     for (int r = p.seqlen_q + tid; r < p.seqlen_q_rounded; r += NTHREADS) LSE[r] = 0.f;
   }
-  // The patch overlays the stages: wait until every wave has finished its last tile.
-  __syncthreads();
+  // The patch overlays the stages; the loop's last barrier already ordered it after all reads.
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(oacc, inv_l, patch, O + (int64_t)q0w * p.o.stride_seq,
                               p.o.stride_seq, p.seqlen_q - q0w, DP, true);
+  FA2_STAMP(3);
 }
 
 }  // namespace fa2
