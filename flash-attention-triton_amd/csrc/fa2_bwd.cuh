@@ -21,6 +21,8 @@
 //    _backward_preprocess_do_o_dot (_triton_kernels_v2.py:532-608).
 #pragma once
 
+#include <type_traits>
+
 #include "fa2_common.cuh"
 
 namespace fa2 {
@@ -462,6 +464,451 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdPa
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   store_transposed_acc<T, DP>(dkacc, p.scale, patch, DK + (int64_t)kv0w * p.dk.stride_seq,
                               p.dk.stride_seq, p.seqlen_k - kv0w, p.headdim, vec);
+}
+
+// ------------------------------------------------------------------------------------------
+// Fast paths (head dimension equal to the padded one, 16-byte aligned rows): the streamed tiles
+// go straight from global memory into swizzled, unpadded LDS with LDS-direct loads, two stages
+// deep, one workgroup barrier per tile.  See fa2_common.cuh for the swizzle and TileLoader.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ void bwd_wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+template <int DP, int BKV>
+struct DqDirectLayout {
+  static constexpr int TILE_ELEMS = BKV * DP;
+  static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;  // K tile then V tile
+  static constexpr int PATCH_ELEMS = kDqWaves * 32 * (DP + 8);
+  static constexpr int TOTAL_ELEMS =
+      (2 * STAGE_ELEMS > PATCH_ELEMS) ? 2 * STAGE_ELEMS : PATCH_ELEMS;
+};
+
+template <typename T, int DP, int BKV>
+__global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const BwdParams p) {
+  using L = DqDirectLayout<DP, BKV>;
+  constexpr int KS = DP / 16, DB = DP / 32;
+  constexpr int BLK = 32;
+  static_assert(BKV == 2 * BLK, "written for 64-row key tiles of two 32-row blocks");
+
+  __shared__ __attribute__((aligned(1024))) short smem[L::TOTAL_ELEMS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 31, h = lane >> 5;
+  const int i16 = lane & 15, g2 = (lane >> 4) & 1;
+
+  const int BH = p.batch * p.nheads;
+  const int bh = blockIdx.x % BH;
+  const int qt = p.n_tiles - 1 - blockIdx.x / BH;
+  const int b = bh / p.nheads, hd = bh % p.nheads;
+  const int q0 = qt * kDqBlockQ;
+  const int q0w = q0 + 32 * wave;
+
+  const short *Q = (const short *)p.q.ptr + b * p.q.stride_batch + hd * p.q.stride_head;
+  const short *K = (const short *)p.k.ptr + b * p.k.stride_batch + hd * p.k.stride_head;
+  const short *V = (const short *)p.v.ptr + b * p.v.stride_batch + hd * p.v.stride_head;
+  const short *DO = (const short *)p.d_o.ptr + b * p.d_o.stride_batch + hd * p.d_o.stride_head;
+  short *DQ = (short *)p.dq.ptr + b * p.dq.stride_batch + hd * p.dq.stride_head;
+
+  const TileLoader<DP, BKV, kDqWaves> kload(K, p.k.stride_seq), vload(V, p.v.stride_seq);
+  const int seqlen_k = p.seqlen_k;
+  const float scale_log2 = p.scale_log2;
+
+  const int kv_end = min(q0 + kDqBlockQ, seqlen_k);
+  const int n_tiles = (kv_end + BKV - 1) / BKV;
+  const int n_mine = min((kv_end + BLK - 1) / BLK, q0w / BLK + 1);  // 32-key blocks of this wave
+  const int n_full = min(q0w + 1, seqlen_k) / BLK;                   // leading blocks without mask
+  const int n_inside = seqlen_k / BKV;
+
+  auto issue_tile = [&](int t) {
+    short *dst = smem + (t & 1) * L::STAGE_ELEMS;
+    if (t < n_inside) {
+      kload.issue(t * BKV, dst);
+      vload.issue(t * BKV, dst + L::TILE_ELEMS);
+    } else {
+      kload.issue_clamped(t * BKV, seqlen_k, dst);
+      vload.issue_clamped(t * BKV, seqlen_k, dst + L::TILE_ELEMS);
+    }
+  };
+  issue_tile(0);
+  if (n_tiles > 1) issue_tile(1);
+
+  // B operands: lane (c, h) holds row q0w + c of Q and of dO, columns 16 ks + 8 h + j.
+  s16x8 qf[KS], gf[KS];
+  float lse2 = 0.f, delta = 0.f;
+  {
+    const int row = q0w + c;
+    const bool ok = row < p.seqlen_q;
+    const short *qp = Q + (int64_t)row * p.q.stride_seq;
+    const short *gp = DO + (int64_t)row * p.d_o.stride_seq;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      qf[ks] = load_chunk(qp, 16 * ks + 8 * h, DP, ok, true);
+      gf[ks] = load_chunk(gp, 16 * ks + 8 * h, DP, ok, true);
+    }
+    if (ok) {
+      lse2 = p.lse[(int64_t)bh * p.seqlen_q_rounded + row] * kLog2e;
+      delta = p.delta[(int64_t)bh * p.seqlen_q_rounded + row];
+    }
+  }
+
+  // Swizzled fragment addresses inside stage 0 (32-bit LDS pointers).
+  const lds_cptr lds0 = to_lds(smem);
+  lds_cptr krow[KS], klo[DB], khi[DB];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) krow[ks] = lds0 + swz_off<DP>(c, 2 * ks + h);
+  {
+    const int rowlo = 4 * h + (i16 >> 2);
+    const int sub = (i16 & 1) * 4;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      const int chunk = 4 * db + 2 * g2 + ((i16 & 3) >> 1);
+      klo[db] = lds0 + swz_off<DP>(rowlo, chunk) + sub;
+      khi[db] = lds0 + swz_off<DP>(rowlo + 8, chunk) + sub;
+    }
+  }
+
+  f32x16 dqacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) dqacc[db][i] = 0.f;
+  const int qrow = q0w + c;
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  bwd_wait_vmem_all();
+  __syncthreads();
+
+  for (int t = 0; t < n_tiles; t++) {
+    const int soff = (t & 1) * L::STAGE_ELEMS;
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++) {
+      const int j = 2 * t + mb;
+      if (j < n_mine) {
+        const int koff = soff + mb * BLK * DP;
+        const int voff = koff + L::TILE_ELEMS;
+        f32x16 s = zero, dp = zero;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) s = Elem<T>::mfma(lds_read_128(krow[ks] + koff), qf[ks], s);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) dp = Elem<T>::mfma(lds_read_128(krow[ks] + voff), gf[ks], dp);
+        const bool need_mask = j >= n_full;
+        f32x16 ds;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          float pr = fast_exp2(s[i] * scale_log2 - lse2);
+          if (need_mask) {
+            const int kv = j * BLK + 8 * (i >> 2) + 4 * h + (i & 3);
+            if (kv > qrow || kv >= seqlen_k) pr = 0.f;
+          }
+          ds[i] = pr * (dp[i] - delta);
+        }
+        f32x8 lo = {ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]};
+        f32x8 hi = {ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]};
+        const s16x8 dsf[2] = {Elem<T>::pack8(lo), Elem<T>::pack8(hi)};
+#pragma unroll
+        for (int ks2 = 0; ks2 < 2; ks2++) {
+#pragma unroll
+          for (int db = 0; db < DB; db++) {
+            s16x4 a0 = lds_read_tr(klo[db] + koff + 16 * ks2 * DP);
+            s16x4 a1 = lds_read_tr(khi[db] + koff + 16 * ks2 * DP);
+            s16x8 a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+            dqacc[db] = Elem<T>::mfma(a, dsf[ks2], dqacc[db]);
+          }
+        }
+      }
+    }
+    // Everyone is done with stage t & 1; tile t+1 (issued one tile ago) has landed.
+    bwd_wait_vmem_all();
+    __syncthreads();
+    if (t + 2 < n_tiles) issue_tile(t + 2);
+  }
+
+  short *patch = smem + wave * 32 * (DP + 8);
+  store_transposed_acc<T, DP>(dqacc, p.scale, patch, DQ + (int64_t)q0w * p.dq.stride_seq,
+                              p.dq.stride_seq, p.seqlen_q - q0w, DP, true);
+}
+
+// dK/dV fast path.  One workgroup per 128 key rows, one wave per 32 of them (K and V fragments in
+// registers); Q and dO tiles of 64 rows stream through three LDS stages (one barrier per tile).
+// The wave runs at one wave per SIMD (dK^T and dV^T alone are 128 accumulator registers), so
+// latency is hidden inside the wave: per 32-row query block the four GEMMs run back to back,
+//     S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS,
+// their A fragments travel through a ring of DP/16 register sets refilled as it is consumed
+// (Q rows -> dO rows -> dO^T -> Q^T -> next block's Q rows), the exponentials are issued under the
+// dP MFMAs and the dS arithmetic under the dV MFMAs.  Blocks on the diagonal (and a ragged last
+// tile) take the same code with the masks switched on.
+template <int DP, int BQ>
+struct DkvDirectLayout {
+  static constexpr int TILE_ELEMS = BQ * DP;
+  // One stage: Q tile, dO tile, then lse*log2e and delta as floats (2 shorts each).
+  static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS + 4 * BQ;
+  static constexpr int STAGES = 3;
+  static constexpr int PATCH_ELEMS = kDkvWaves * 32 * (DP + 8);
+  static constexpr int TOTAL_ELEMS =
+      (STAGES * STAGE_ELEMS > PATCH_ELEMS) ? STAGES * STAGE_ELEMS : PATCH_ELEMS;
+};
+
+template <typename T, int DP, int BQ>
+__global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(const BwdParams p) {
+  using L = DkvDirectLayout<DP, BQ>;
+  constexpr int KS = DP / 16, DB = DP / 32;
+  constexpr int NTHREADS = 64 * kDkvWaves;
+  static_assert(BQ == 64 && KS == 2 * DB, "schedule is written for 64-row query tiles of two blocks");
+  static_assert(BQ <= NTHREADS, "one thread per row loads lse and delta");
+  static_assert((L::STAGE_ELEMS * 2) % 256 == 0, "stages must start on a 256-byte LDS bank line");
+
+  __shared__ __attribute__((aligned(1024))) short smem[L::TOTAL_ELEMS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 31, h = lane >> 5;
+  const int i16 = lane & 15, g2 = (lane >> 4) & 1;
+
+  // Key tile 0 has the longest query range: issue tiles in ascending order (heaviest first).
+  const int BH = p.batch * p.nheads;
+  const int bh = blockIdx.x % BH;
+  const int kt = blockIdx.x / BH;
+  const int b = bh / p.nheads, hd = bh % p.nheads;
+  const int kv0 = kt * kDkvBlockKV;
+  const int kv0w = kv0 + 32 * wave;
+
+  const short *Q = (const short *)p.q.ptr + b * p.q.stride_batch + hd * p.q.stride_head;
+  const short *K = (const short *)p.k.ptr + b * p.k.stride_batch + hd * p.k.stride_head;
+  const short *V = (const short *)p.v.ptr + b * p.v.stride_batch + hd * p.v.stride_head;
+  const short *DO = (const short *)p.d_o.ptr + b * p.d_o.stride_batch + hd * p.d_o.stride_head;
+  short *DK = (short *)p.dk.ptr + b * p.dk.stride_batch + hd * p.dk.stride_head;
+  short *DV = (short *)p.dv.ptr + b * p.dv.stride_batch + hd * p.dv.stride_head;
+  const float *LSE = p.lse + (int64_t)bh * p.seqlen_q_rounded;
+  const float *DELTA = p.delta + (int64_t)bh * p.seqlen_q_rounded;
+
+  const TileLoader<DP, BQ, kDkvWaves> qload(Q, p.q.stride_seq), gload(DO, p.d_o.stride_seq);
+  const int seqlen_q = p.seqlen_q;
+  const float scale_log2 = p.scale_log2;
+
+  // First query tile that can see this key tile (row >= col), aligned down to BQ.
+  const int q_begin = (kv0 / BQ) * BQ;
+  const int n_tiles = (seqlen_q > q_begin) ? (seqlen_q - q_begin + BQ - 1) / BQ : 0;
+  const int n_inside = (seqlen_q - q_begin) / BQ;  // tiles whose every row exists
+  // Tiles that touch the diagonal of this key tile (their blocks need the causal mask).
+  const int n_diag = min(n_tiles, (kv0 + kDkvBlockKV - q_begin + BQ - 1) / BQ);
+
+  auto issue_tile = [&](int t) {
+    short *dst = smem + (t % L::STAGES) * L::STAGE_ELEMS;
+    const int row0 = q_begin + t * BQ;
+    if (t < n_inside) {
+      qload.issue(row0, dst);
+      gload.issue(row0, dst + L::TILE_ELEMS);
+    } else {
+      qload.issue_clamped(row0, seqlen_q, dst);
+      gload.issue_clamped(row0, seqlen_q, dst + L::TILE_ELEMS);
+    }
+  };
+  // lse*log2e and delta of a tile go through registers into the stage's statistics area (rows
+  // beyond the sequence get 0: their probabilities are zeroed by the row mask).
+  float lse_reg = 0.f, delta_reg = 0.f;
+  auto load_stats = [&](int t) {
+    if (tid < BQ) {
+      const int row = q_begin + t * BQ + tid;
+      const bool ok = row < seqlen_q;
+      lse_reg = ok ? LSE[row] * kLog2e : 0.f;
+      delta_reg = ok ? DELTA[row] : 0.f;
+    }
+  };
+  auto store_stats = [&](int t) {
+    float *sl = reinterpret_cast<float *>(smem + (t % L::STAGES) * L::STAGE_ELEMS + 2 * L::TILE_ELEMS);
+    if (tid < BQ) {
+      sl[tid] = lse_reg;
+      sl[BQ + tid] = delta_reg;
+    }
+  };
+#pragma unroll
+  for (int t = 0; t < L::STAGES; t++) {
+    if (t < n_tiles) {
+      issue_tile(t);
+      load_stats(t);
+      store_stats(t);
+    }
+  }
+
+  // B operands: lane (c, h) holds row kv0w + c of K and of V, columns 16 ks + 8 h + j.
+  s16x8 kf[KS], vf[KS];
+  {
+    const int row = kv0w + c;
+    const bool ok = row < p.seqlen_k;
+    const short *kp = K + (int64_t)row * p.k.stride_seq;
+    const short *vp = V + (int64_t)row * p.v.stride_seq;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      kf[ks] = load_chunk(kp, 16 * ks + 8 * h, DP, ok, true);
+      vf[ks] = load_chunk(vp, 16 * ks + 8 * h, DP, ok, true);
+    }
+  }
+
+  // Swizzled fragment addresses (32-bit LDS pointers) into the current tile's stage; the dO tile
+  // sits TILE_ELEMS after the Q tile.  qnext runs one block ahead (for the ring prefetch).
+  const lds_cptr lds0 = to_lds(smem);
+  lds_cptr qnext[KS], qrow[KS], qlo[DB], qhi[DB];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) {
+    qrow[ks] = lds0 + swz_off<DP>(c, 2 * ks + h);
+    qnext[ks] = qrow[ks];
+  }
+  {
+    const int rowlo = 4 * h + (i16 >> 2);
+    const int sub = (i16 & 1) * 4;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      const int chunk = 4 * db + 2 * g2 + ((i16 & 3) >> 1);
+      qlo[db] = lds0 + swz_off<DP>(rowlo, chunk) + sub;
+      qhi[db] = lds0 + swz_off<DP>(rowlo + 8, chunk) + sub;
+    }
+  }
+  const __attribute__((address_space(3))) float *stat =
+      reinterpret_cast<const __attribute__((address_space(3))) float *>(lds0 + 2 * L::TILE_ELEMS) + 4 * h;
+
+  f32x16 dkacc[DB], dvacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      dkacc[db][i] = 0.f;
+      dvacc[db][i] = 0.f;
+    }
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const int kvcol = kv0w + c;
+
+  bwd_wait_vmem_all();
+  __syncthreads();
+
+  // Ring of A fragments, preloaded with the Q rows of block 0.
+  s16x8 ring[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) ring[ks] = lds_read_128(qrow[ks]);
+
+  // One 32-row query block.  HALF selects the half-tile; MASKED switches the causal/row masks on.
+  auto block = [&](int qb, auto half_tag, auto masked_tag) {
+    constexpr int HALF = decltype(half_tag)::value;
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    constexpr int QOFF = HALF * 32 * DP;          // Q rows of this block inside the tile
+    constexpr int GOFF = QOFF + L::TILE_ELEMS;    // dO rows of this block
+    typedef const __attribute__((address_space(3))) f32x4 *stat4_ptr;
+
+    // ---- S = Q K^T (ring: Q rows -> dO rows); statistics of the 16 rows this lane holds -----
+    f32x16 s = zero, dp = zero;
+    f32x4 l4[4], d4[4];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      s = Elem<T>::mfma(ring[ks], kf[ks], s);
+      ring[ks] = lds_read_128(qrow[ks] + GOFF);
+      constexpr int PER = (4 + KS - 1) / KS;  // row groups of four fetched per unit
+#pragma unroll
+      for (int u = 0; u < PER; u++) {
+        const int g = ks * PER + u;
+        if (g < 4) {
+          l4[g] = *reinterpret_cast<stat4_ptr>(stat + 32 * HALF + 8 * g);
+          d4[g] = *reinterpret_cast<stat4_ptr>(stat + BQ + 32 * HALF + 8 * g);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- dP = dO V^T (ring: dO rows -> dO^T); exponentials under the MFMAs -------------------
+    f32x16 pr;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      dp = Elem<T>::mfma(ring[ks], vf[ks], dp);
+      {
+        s16x4 a0 = lds_read_tr(qlo[ks % DB] + GOFF + 16 * (ks / DB) * DP);
+        s16x4 a1 = lds_read_tr(qhi[ks % DB] + GOFF + 16 * (ks / DB) * DP);
+        ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+#pragma unroll
+      for (int u = 0; u < 16 / KS; u++) {
+        const int i = (16 / KS) * ks + u;
+        float x = fast_exp2(s[i] * scale_log2 - l4[i >> 2][i & 3]);
+        if (MASKED) {
+          const int qr = qb + 8 * (i >> 2) + 4 * h + (i & 3);
+          if (kvcol > qr || qr >= seqlen_q) x = 0.f;
+        }
+        pr[i] = x;
+      }
+      asm volatile("" : "+v"(pr));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    f32x8 plo = {pr[0], pr[1], pr[2], pr[3], pr[4], pr[5], pr[6], pr[7]};
+    f32x8 phi = {pr[8], pr[9], pr[10], pr[11], pr[12], pr[13], pr[14], pr[15]};
+    const s16x8 pf[2] = {Elem<T>::pack8(plo), Elem<T>::pack8(phi)};
+    // ---- dV^T += dO^T P (ring: dO^T -> Q^T); dS arithmetic under the MFMAs --------------------
+    f32x16 ds;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      dvacc[ks % DB] = Elem<T>::mfma(ring[ks], pf[ks / DB], dvacc[ks % DB]);
+      {
+        s16x4 a0 = lds_read_tr(qlo[ks % DB] + QOFF + 16 * (ks / DB) * DP);
+        s16x4 a1 = lds_read_tr(qhi[ks % DB] + QOFF + 16 * (ks / DB) * DP);
+        ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+#pragma unroll
+      for (int u = 0; u < 16 / KS; u++) {
+        const int i = (16 / KS) * ks + u;
+        ds[i] = pr[i] * (dp[i] - d4[i >> 2][i & 3]);
+      }
+      asm volatile("" : "+v"(ds));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    f32x8 dlo = {ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]};
+    f32x8 dhi = {ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]};
+    const s16x8 dsf[2] = {Elem<T>::pack8(dlo), Elem<T>::pack8(dhi)};
+    // ---- dK^T += Q^T dS (ring: Q^T -> Q rows of the next block) --------------------------------
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      dkacc[ks % DB] = Elem<T>::mfma(ring[ks], dsf[ks / DB], dkacc[ks % DB]);
+      ring[ks] = lds_read_128(qnext[ks] + (HALF == 0 ? 32 * DP : 0));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  auto tile = [&](int t, auto masked_tag) {
+    const int qt0 = q_begin + t * BQ;
+    // qnext -> next tile's stage before the second block prefetches from it.
+    const int d = ((t + 1) % L::STAGES == 0) ? -(L::STAGES - 1) * L::STAGE_ELEMS : L::STAGE_ELEMS;
+    block(qt0, std::integral_constant<int, 0>{}, masked_tag);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qnext[ks] += d;
+    block(qt0 + 32, std::integral_constant<int, 1>{}, masked_tag);
+    // Tile t+3's statistics were loaded one tile ago; their stage was freed by the last barrier.
+    if (t >= 1 && t + 2 < n_tiles) store_stats(t + 2);
+    // Everyone is done with stage t % 3; tile t+2 (issued one tile ago) has landed.
+    bwd_wait_vmem_all();
+    __syncthreads();
+    if (t + 3 < n_tiles) {
+      issue_tile(t + 3);
+      load_stats(t + 3);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qrow[ks] += d;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      qlo[db] += d;
+      qhi[db] += d;
+    }
+    stat += d / 2;  // float elements
+  };
+
+  int t = 0;
+  for (; t < n_diag; t++) tile(t, std::true_type{});
+  for (; t < n_inside; t++) tile(t, std::false_type{});
+  for (; t < n_tiles; t++) tile(t, std::true_type{});
+
+  short *patch = smem + wave * 32 * (DP + 8);
+  store_transposed_acc<T, DP>(dvacc, 1.0f, patch, DV + (int64_t)kv0w * p.dv.stride_seq,
+                              p.dv.stride_seq, p.seqlen_k - kv0w, DP, true);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  store_transposed_acc<T, DP>(dkacc, p.scale, patch, DK + (int64_t)kv0w * p.dk.stride_seq,
+                              p.dk.stride_seq, p.seqlen_k - kv0w, DP, true);
 }
 
 }  // namespace fa2

@@ -134,6 +134,14 @@ void launch_fwd(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
 template <typename T>
 void launch_dq(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
   dim3 block(64 * fa2::kDqWaves);
+  if (p.vec && p.headdim == dp && dp != 96 && direct_ok(p.k) && direct_ok(p.v)) {
+    switch (dp) {
+      case 32: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 32, kDqBlockKV>), grid, block, 0, s, p); break;
+      case 64: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 64, kDqBlockKV>), grid, block, 0, s, p); break;
+      default: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 128, kDqBlockKV>), grid, block, 0, s, p); break;
+    }
+    return;
+  }
   switch (dp) {
     case 32: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 32, kDqBlockKV>), grid, block, 0, s, p); break;
     case 64: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 64, kDqBlockKV>), grid, block, 0, s, p); break;
@@ -145,6 +153,14 @@ void launch_dq(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
 template <typename T>
 void launch_dkdv(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
   dim3 block(64 * fa2::kDkvWaves);
+  if (p.vec && p.headdim == dp && dp != 96 && direct_ok(p.q) && direct_ok(p.d_o)) {
+    switch (dp) {
+      case 32: hipLaunchKernelGGL((fa2::bwd_dkdv_direct_kernel<T, 32, kDkvBlockQ>), grid, block, 0, s, p); break;
+      case 64: hipLaunchKernelGGL((fa2::bwd_dkdv_direct_kernel<T, 64, kDkvBlockQ>), grid, block, 0, s, p); break;
+      default: hipLaunchKernelGGL((fa2::bwd_dkdv_direct_kernel<T, 128, kDkvBlockQ>), grid, block, 0, s, p); break;
+    }
+    return;
+  }
   switch (dp) {
     case 32: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 32, kDkvBlockQ>), grid, block, 0, s, p); break;
     case 64: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 64, kDkvBlockQ>), grid, block, 0, s, p); break;
