@@ -29,6 +29,17 @@ sys.path.insert(0, str(ROOT))
 
 # Published dense peaks of MI355X.
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}
+CALIBRATION_BYTES = 256 << 20
+# HBM bytes per launch on workload C3 (bf16), read off rocprofv3's FETCH_SIZE / WRITE_SIZE counters
+# and scaled by what the same counters read for the --traffic-calibration copy (x2.000 / x1.000);
+# the summary sits in profiles/fwd_bwd_kernels_c3_bf16_hbm_traffic.txt.  Counters cannot be read
+# from inside the process, so other workloads report null.
+MEASURED_TRAFFIC_BYTES = {
+    ("C3", "fwd"): 771.7e6,
+    ("C3", "bwd_dkdv"): 880.3e6,
+    ("C3", "bwd_dq"): 624.6e6,
+    ("C3", "bwd_preprocess"): 135.3e6,
+}
 PEAK_HBM_GBS = 8000.0
 METRIC = "causal attn TFLOP/s fwd & fwd+bwd (bf16, D=128) and % of MFMA peak, 1 GPU"
 
@@ -90,21 +101,30 @@ def _kernel_legs(capi, w, q, k, v, d_o, iters: int):
     torch.cuda.synchronize()
     results["fwd"] = _event_time_ms(fwd, iters)
     results["bwd_preprocess"] = _event_time_ms(pre, iters)
-    for det in (1, 0):
-        ws_bytes = lib.fa2_bwd_workspace_bytes(b, h, n, n, d, det, capi.FA2_CONFIG_AUTO)
-        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=q.device)
+    ws_bytes = lib.fa2_bwd_workspace_bytes(b, h, n, n, d, 0, capi.FA2_CONFIG_AUTO)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=q.device)
 
-        def bwd(det=det, ws=ws):
-            capi.check(lib.fa2_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), d_o.data_ptr(),
-                                   lse.data_ptr(), delta.data_ptr(), ws.data_ptr(),
-                                   dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-                                   b, h, n, n, d, n_r, *s3(q), *s3(k), *s3(v), *s3(d_o),
-                                   *s3(dq), *s3(dk), *s3(dv), scale, dtype, det,
-                                   capi.FA2_CONFIG_AUTO, stream), "fa2_bwd")
+    def bwd(det, want_dq=True, want_dkdv=True):
+        capi.check(lib.fa2_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), d_o.data_ptr(),
+                               lse.data_ptr(), delta.data_ptr(), ws.data_ptr(),
+                               dq.data_ptr() if want_dq else None,
+                               dk.data_ptr() if want_dkdv else None,
+                               dv.data_ptr() if want_dkdv else None,
+                               b, h, n, n, d, n_r, *s3(q), *s3(k), *s3(v), *s3(d_o),
+                               *s3(dq), *s3(dk), *s3(dv), scale, dtype, det,
+                               capi.FA2_CONFIG_AUTO, stream), "fa2_bwd")
 
-        bwd()
+    legs = {
+        "bwd_deterministic": lambda: bwd(1),
+        "bwd_sequence_parallel": lambda: bwd(0),
+        # One kernel each: NULL outputs switch the other kernel off.
+        "bwd_dkdv": lambda: bwd(0, want_dq=False),
+        "bwd_dq": lambda: bwd(0, want_dkdv=False),
+    }
+    for name, fn in legs.items():
+        fn()
         torch.cuda.synchronize()
-        results["bwd_deterministic" if det else "bwd_sequence_parallel"] = _event_time_ms(bwd, iters)
+        results[name] = _event_time_ms(fn, iters)
     return results
 
 
@@ -139,8 +159,11 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--deterministic", action="store_true", help="time the deterministic backward in the step")
-    ap.add_argument("--cpu-heads", type=int, default=2, help="(batch, head) slices in the CPU baseline sample")
+    ap.add_argument("--cpu-heads", type=int, default=64, help="(batch, head) slices in the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="also launch a plain 256 MiB -> 256 MiB elementwise copy three times, so a hardware-"
+                         "counter run of this command holds a kernel of known HBM traffic to scale by")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -198,32 +221,33 @@ def main() -> int:
     # Per-kernel legs through the C ABI, timed with HIP events on the launch stream.
     legs = _kernel_legs(capi, w, q.detach(), k.detach(), v.detach(), d_o, max(args.steps, 5))
     leg_ms = {name: statistics.mean(ts) for name, ts in legs.items()}
-    # Algorithmic FLOPs: the forward owns 2 GEMMs (1 x fwd_flops), the backward 5 (2.5 x).
+    # FLOPs per launch, counted in causal GEMMs of fwd_flops / 2 each: the forward kernel owns 2
+    # (S, PV), the dK/dV kernel 4 (S, dP, dV, dK), the dQ kernel 3 (S, dP, dQ).  The whole backward
+    # is priced at the conventional 5 (2.5 x forward) although the two kernels execute 7.
+    kernels = {
+        "fwd": ("fwd_direct_kernel (fa2_fwd)", 1.0 * w.fwd_flops),
+        "bwd_dkdv": ("bwd_dkdv_direct_kernel (fa2_bwd, dK/dV half)", 2.0 * w.fwd_flops),
+        "bwd_dq": ("bwd_dq_direct_kernel (fa2_bwd, dQ half)", 1.5 * w.fwd_flops),
+    }
+    dominant = max(kernels, key=lambda name: leg_ms[name])
+
+    def mfma_roofline(name):
+        label, flops = kernels[name]
+        achieved = flops / (leg_ms[name] * 1e-3) / 1e12
+        return {"kernel": label, "bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, name)),
+                "flops_per_launch": flops,
+                "avg_launch_ms": leg_ms[name]}
+
+    roofline = mfma_roofline(dominant)
     bwd_leg = "bwd_deterministic" if det else "bwd_sequence_parallel"
-    dominant = "fwd" if leg_ms["fwd"] >= leg_ms[bwd_leg] else bwd_leg
-    dom_flops = w.fwd_flops if dominant == "fwd" else w.bwd_flops
-    achieved = dom_flops / (leg_ms[dominant] * 1e-3) / 1e12
-    roofline = {
-        "kernel": "fa2_fwd (fwd_kernel)" if dominant == "fwd" else f"fa2_bwd ({bwd_leg}: bwd_dkdv_kernel + bwd_dq_kernel)",
-        "bound": "mfma",
-        "achieved": achieved,
-        "peak": peak,
-        "unit": "TFLOP/s",
-        "frac": achieved / peak,
-        "traffic": None,
-        "avg_launch_ms": leg_ms[dominant],
-    }
-    fwd_roofline = {
-        "kernel": "fa2_fwd (fwd_kernel)", "bound": "mfma",
-        "achieved": w.fwd_flops / (leg_ms["fwd"] * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
-        "frac": w.fwd_flops / (leg_ms["fwd"] * 1e-3) / 1e12 / peak, "traffic": None,
-        "avg_launch_ms": leg_ms["fwd"],
-    }
+    bwd_tflops = w.bwd_flops / (leg_ms[bwd_leg] * 1e-3) / 1e12
     pre_bytes = 2.0 * w.batch * w.nheads * w.seqlen * w.headdim * 2 + w.batch * w.nheads * w.seqlen * 4
     pre_roofline = {
         "kernel": "fa2_bwd_preprocess (bwd_preprocess_kernel)", "bound": "hbm",
         "achieved": pre_bytes / (leg_ms["bwd_preprocess"] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-        "frac": pre_bytes / (leg_ms["bwd_preprocess"] * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+        "frac": pre_bytes / (leg_ms["bwd_preprocess"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, "bwd_preprocess")), "bytes_per_launch": pre_bytes,
         "avg_launch_ms": leg_ms["bwd_preprocess"],
     }
 
@@ -256,10 +280,22 @@ def main() -> int:
                    "compute_units": props.multi_processor_count,
                    "clock_mhz": getattr(props, "clock_rate", 0) / 1e3},
         "roofline": roofline,
-        "roofline_fwd": fwd_roofline,
+        "roofline_fwd": mfma_roofline("fwd"),
+        "roofline_bwd_dkdv": mfma_roofline("bwd_dkdv"),
+        "roofline_bwd_dq": mfma_roofline("bwd_dq"),
+        "bwd_tflops_algorithmic": bwd_tflops,
+        "bwd_frac_of_peak": bwd_tflops / peak,
         "roofline_bwd_preprocess": pre_roofline,
         "kernel_ms": leg_ms,
     }
+    if args.traffic_calibration:
+        src = torch.ones(CALIBRATION_BYTES // 4, device=dev, dtype=torch.float32)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        line["traffic_calibration"] = {"kernel": "torch elementwise mul (fp32, out=)",
+                                       "read_bytes": CALIBRATION_BYTES, "write_bytes": CALIBRATION_BYTES}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(w, workloads, args.cpu_heads)
     print(json.dumps(line))

@@ -318,11 +318,17 @@ int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const 
   p.dq = tensor(dq, dq_sb, dq_sh, dq_ss);
   p.dk = tensor(dk, dk_sb, dk_sh, dk_ss);
   p.dv = tensor(dv, dv_sb, dv_sh, dv_ss);
+  // A caller that needs only part of the gradient passes NULL for the rest: dq == NULL skips the
+  // dQ kernel, dk == dv == NULL skips the dK/dV kernel.  dk and dv come from one kernel, so they
+  // are given or omitted together.
+  const bool want_dq = dq != nullptr;
+  const bool want_dkdv = dk != nullptr || dv != nullptr;
+  if (!want_dq && !want_dkdv) return fail(FA2_ERR_NULL_POINTER, "dq, dk and dv are all NULL");
   if ((rc = check_tensor("q", p.q)) || (rc = check_tensor("k", p.k)) ||
-      (rc = check_tensor("v", p.v)) || (rc = check_tensor("d_o", p.d_o)) ||
-      (rc = check_tensor("dq", p.dq)) || (rc = check_tensor("dk", p.dk)) ||
-      (rc = check_tensor("dv", p.dv)))
+      (rc = check_tensor("v", p.v)) || (rc = check_tensor("d_o", p.d_o)))
     return rc;
+  if (want_dq && (rc = check_tensor("dq", p.dq))) return rc;
+  if (want_dkdv && ((rc = check_tensor("dk", p.dk)) || (rc = check_tensor("dv", p.dv)))) return rc;
   if (lse == nullptr) return fail(FA2_ERR_NULL_POINTER, "lse is NULL");
   if (delta == nullptr) return fail(FA2_ERR_NULL_POINTER, "delta is NULL");
   if (!(softmax_scale > 0.f) || !std::isfinite(softmax_scale))
@@ -341,14 +347,14 @@ int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const 
   p.scale = softmax_scale;
   p.scale_log2 = softmax_scale * fa2::kLog2e;
   p.vec = vec_ok(p.q, headdim) && vec_ok(p.k, headdim) && vec_ok(p.v, headdim) &&
-          vec_ok(p.d_o, headdim) && vec_ok(p.dq, headdim) && vec_ok(p.dk, headdim) &&
-          vec_ok(p.dv, headdim);
+          vec_ok(p.d_o, headdim) && (!want_dq || vec_ok(p.dq, headdim)) &&
+          (!want_dkdv || (vec_ok(p.dk, headdim) && vec_ok(p.dv, headdim)));
 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const int dp = kTable[cfg].headdim_padded;
   const int64_t bh = (int64_t)batch * nheads;
 
-  {  // dK, dV
+  if (want_dkdv) {  // dK, dV
     fa2::BwdParams pk = p;
     pk.n_tiles = (seqlen_k + fa2::kDkvBlockKV - 1) / fa2::kDkvBlockKV;
     const int64_t nwg = pk.n_tiles * bh;
@@ -360,7 +366,7 @@ int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const 
       launch_dkdv<_Float16>(dp, pk, grid, s);
     if ((rc = launch_status("fa2_bwd dK/dV launch"))) return rc;
   }
-  {  // dQ
+  if (want_dq) {  // dQ
     fa2::BwdParams pq = p;
     pq.n_tiles = (seqlen_q + fa2::kDqBlockQ - 1) / fa2::kDqBlockQ;
     const int64_t nwg = pq.n_tiles * bh;

@@ -142,6 +142,10 @@ size_t fa2_bwd_workspace_bytes(int batch, int nheads, int seqlen_q, int seqlen_k
  *                       (sequence-parallel mode); low-order bits can differ between runs.
  * `workspace` must hold fa2_bwd_workspace_bytes(...) bytes (may be NULL when that is 0); the
  * library clears what it needs.
+ * dK/dV and dQ are computed by two kernels launched back to back on `stream`.  A caller that
+ * needs only part of the gradient (or wants to time one kernel) may pass dq == NULL to skip the
+ * dQ kernel, or dk == dv == NULL to skip the dK/dV kernel; dk and dv are given or omitted
+ * together, and at least one of the two groups must be present.
  */
 int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o,
             const float *lse, const float *delta, void *workspace,

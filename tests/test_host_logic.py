@@ -113,6 +113,15 @@ def test_backward_entry_points_reject_bad_arguments(capi):
                      0.125, capi.FA2_DTYPE_F16, 1, capi.FA2_CONFIG_AUTO, None)
     assert lib.fa2_status_string(rc).decode() == "FA2_ERR_BAD_SHAPE"
     assert lib.fa2_bwd_workspace_bytes(2, 4, 512, 512, 64, 1, capi.FA2_CONFIG_AUTO) == 0
+    # Either gradient group may be omitted, but not both, and dk/dv only together.
+    rc = lib.fa2_bwd(16, 16, 16, 16, 16, 16, None, None, None, None, 1, 1, 8, 8, 64, 128, *(st * 7),
+                     0.125, capi.FA2_DTYPE_F16, 1, capi.FA2_CONFIG_AUTO, None)
+    assert lib.fa2_status_string(rc).decode() == "FA2_ERR_NULL_POINTER"
+    assert "all NULL" in lib.fa2_last_error_string().decode()
+    rc = lib.fa2_bwd(16, 16, 16, 16, 16, 16, None, 16, 16, None, 1, 1, 8, 8, 64, 128, *(st * 7),
+                     0.125, capi.FA2_DTYPE_F16, 1, capi.FA2_CONFIG_AUTO, None)
+    assert lib.fa2_status_string(rc).decode() == "FA2_ERR_NULL_POINTER"
+    assert "dv" in lib.fa2_last_error_string().decode()
 
 
 def test_missing_library_fails_loudly(capi, monkeypatch, tmp_path):

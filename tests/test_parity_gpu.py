@@ -128,6 +128,50 @@ def test_lse_and_delta_match_oracle(fa2_module, capi, name):
     _assert_close("delta vs exact", delta[..., :nq], g["delta"], atol=3e-2, rtol=1e-2)
 
 
+def test_partial_gradients_through_c_abi(fa2_module, capi):
+    """dq == NULL or dk == dv == NULL runs one of the two backward kernels; what it writes is
+    bit-identical to the full call and the omitted outputs are left untouched."""
+    g = golden_io.load(golden_io.NAMES[0])
+    cfg = fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC
+    q, k, v, d_o = (g[x].cuda() for x in ("q", "k", "v", "d_o"))
+    out, lse, scale = fa2_module._flash_attention_forward(
+        q, k, v, g["scale"], cfg.block_rows_size, cfg.block_cols_size, cfg.min_block_headdim,
+        cfg.max_headdim, cfg.seqlen_cache_divisor, cfg.min_warps, cfg.max_warps, cfg.num_stages)
+    b, h, nq, d = q.shape
+    nk = k.shape[2]
+    n_r = lse.shape[-1]
+    lib = capi.load()
+    s3 = fa2_module._strides3
+    dtype = fa2_module._COMPUTE_DTYPES[q.dtype]
+    stream = torch.cuda.current_stream().cuda_stream
+    delta = torch.empty_like(lse)
+    capi.check(lib.fa2_bwd_preprocess(out.data_ptr(), d_o.data_ptr(), delta.data_ptr(), b, h, nq, d, n_r,
+                                      *s3(out), *s3(d_o), dtype, stream), "fa2_bwd_preprocess")
+
+    def run(want_dq, want_dkdv):
+        dq, dk, dv = (torch.full_like(t, 7.0) for t in (q, k, v))
+        capi.check(lib.fa2_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), d_o.data_ptr(), lse.data_ptr(),
+                               delta.data_ptr(), None,
+                               dq.data_ptr() if want_dq else None,
+                               dk.data_ptr() if want_dkdv else None,
+                               dv.data_ptr() if want_dkdv else None,
+                               b, h, nq, nk, d, n_r, *s3(q), *s3(k), *s3(v), *s3(d_o),
+                               *s3(dq), *s3(dk), *s3(dv), scale, dtype, 1, capi.FA2_CONFIG_AUTO, stream),
+                   "fa2_bwd")
+        torch.cuda.synchronize()
+        return dq, dk, dv
+
+    full = run(True, True)
+    only_dq = run(True, False)
+    only_dkdv = run(False, True)
+    assert torch.equal(only_dq[0], full[0])
+    assert torch.equal(only_dkdv[1], full[1]) and torch.equal(only_dkdv[2], full[2])
+    assert (only_dq[1] == 7).all() and (only_dq[2] == 7).all() and (only_dkdv[0] == 7).all()
+    _assert_close("dq", full[0], g["dq"])
+    _assert_close("dk", full[1], g["dk"])
+    _assert_close("dv", full[2], g["dv"])
+
+
 # ------------------------------------------------------------------------- BASELINE configurations at full size
 def _workload_case(workloads, name):
     w = workloads.WORKLOADS[name]
