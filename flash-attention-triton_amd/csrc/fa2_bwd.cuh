@@ -659,6 +659,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(cons
   static_assert((L::STAGE_ELEMS * 2) % 256 == 0, "stages must start on a 256-byte LDS bank line");
 
   __shared__ __attribute__((aligned(1024))) short smem[L::TOTAL_ELEMS];
+  FA2_STAMP(0);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -723,14 +724,12 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(cons
       sl[BQ + tid] = delta_reg;
     }
   };
+  // Prologue: every global load of the first three tiles and of this wave's K and V rows is
+  // issued before anything waits, so that the workgroup pays one memory latency, not one per
+  // tile.
 #pragma unroll
-  for (int t = 0; t < L::STAGES; t++) {
-    if (t < n_tiles) {
-      issue_tile(t);
-      load_stats(t);
-      store_stats(t);
-    }
-  }
+  for (int t = 0; t < L::STAGES; t++)
+    if (t < n_tiles) issue_tile(t);
 
   // B operands: lane (c, h) holds row kv0w + c of K and of V, columns 16 ks + 8 h + j.
   s16x8 kf[KS], vf[KS];
@@ -743,6 +742,21 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(cons
     for (int ks = 0; ks < KS; ks++) {
       kf[ks] = load_chunk(kp, 16 * ks + 8 * h, DP, ok, true);
       vf[ks] = load_chunk(vp, 16 * ks + 8 * h, DP, ok, true);
+    }
+  }
+  {
+    float l3[L::STAGES], d3[L::STAGES];
+#pragma unroll
+    for (int t = 0; t < L::STAGES; t++) {
+      load_stats(t);  // rows beyond the sequence (and tiles beyond the last) read as 0
+      l3[t] = lse_reg;
+      d3[t] = delta_reg;
+    }
+#pragma unroll
+    for (int t = 0; t < L::STAGES; t++) {
+      lse_reg = l3[t];
+      delta_reg = d3[t];
+      store_stats(t);
     }
   }
 
@@ -782,6 +796,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(cons
   bwd_wait_vmem_all();
   __syncthreads();
 
+  FA2_STAMP(1);
   // Ring of A fragments, preloaded with the Q rows of block 0.
   s16x8 ring[KS];
 #pragma unroll
@@ -900,6 +915,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(cons
   for (; t < n_diag; t++) tile(t, std::true_type{});
   for (; t < n_inside; t++) tile(t, std::false_type{});
   for (; t < n_tiles; t++) tile(t, std::true_type{});
+  FA2_STAMP(2);
 
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(dvacc, 1.0f, patch, DV + (int64_t)kv0w * p.dv.stride_seq,
@@ -909,6 +925,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(cons
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   store_transposed_acc<T, DP>(dkacc, p.scale, patch, DK + (int64_t)kv0w * p.dk.stride_seq,
                               p.dk.stride_seq, p.seqlen_k - kv0w, DP, true);
+  FA2_STAMP(3);
 }
 
 }  // namespace fa2

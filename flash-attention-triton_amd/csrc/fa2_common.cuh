@@ -211,6 +211,14 @@ __device__ __forceinline__ void store_transposed_acc(const f32x16 (&acc)[DP / 32
   }
 }
 
+#ifdef FA2_WG_STAMPS
+// Debug build only: wall-clock (100 MHz) stamps per workgroup: start, loop start, loop end, end.
+__device__ long long fa2_wg_stamps[8192][4];
+#define FA2_STAMP(slot) do { if (threadIdx.x == 0 && blockIdx.x < 8192) fa2_wg_stamps[blockIdx.x][slot] = wall_clock64(); } while (0)
+#else
+#define FA2_STAMP(slot) do {} while (0)
+#endif
+
 }  // namespace fa2
 
 // ------------------------------------------------------------------------------------------

@@ -294,13 +294,6 @@ __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0
 // Scheduling-group masks of __builtin_amdgcn_sched_group_barrier.
 constexpr int kSgValu = 0x002, kSgMfma = 0x008, kSgDsRead = 0x100, kSgTrans = 0x400;
 
-#ifdef FA2_WG_STAMPS
-// Debug build only: wall-clock (100 MHz) stamps per workgroup: start, loop start, loop end, end.
-__device__ long long fa2_wg_stamps[8192][4];
-#define FA2_STAMP(slot) do { if (threadIdx.x == 0 && blockIdx.x < 8192) fa2_wg_stamps[blockIdx.x][slot] = wall_clock64(); } while (0)
-#else
-#define FA2_STAMP(slot) do {} while (0)
-#endif
 
 template <typename T, int DP, int BKV>
 __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const FwdParams p) {
