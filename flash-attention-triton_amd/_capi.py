@@ -17,7 +17,7 @@ ABI_VERSION = 1
 FA2_DTYPE_F16 = 0
 FA2_DTYPE_BF16 = 1
 FA2_CONFIG_AUTO = -1
-FA2_MAX_HEADDIM = 128
+FA2_MAX_HEADDIM = 256
 
 _i, _i64, _f, _p = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 

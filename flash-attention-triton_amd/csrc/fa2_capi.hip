@@ -37,6 +37,8 @@ const fa2_config_info kTable[] = {
     {1, 64, fa2::kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, fa2::kDkvBlockKV, 4, fa2::kDqBlockQ, kDqBlockKV, 4},
     {2, 96, fa2::kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, fa2::kDkvBlockKV, 4, fa2::kDqBlockQ, kDqBlockKV, 4},
     {3, 128, fa2::kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, fa2::kDkvBlockKV, 4, fa2::kDqBlockQ, kDqBlockKV, 4},
+    {4, 192, fa2::kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, fa2::kDkvBlockKV, 4, fa2::kDqBlockQ, kDqBlockKV, 4},
+    {5, 256, fa2::kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, fa2::kDkvBlockKV, 4, fa2::kDqBlockQ, kDqBlockKV, 4},
 };
 constexpr int kTableRows = sizeof(kTable) / sizeof(kTable[0]);
 
@@ -106,7 +108,9 @@ void launch_fwd_v(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
     case 32: hipLaunchKernelGGL((fa2::fwd_kernel<T, 32, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
     case 64: hipLaunchKernelGGL((fa2::fwd_kernel<T, 64, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
     case 96: hipLaunchKernelGGL((fa2::fwd_kernel<T, 96, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fa2::fwd_kernel<T, 128, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
+    case 128: hipLaunchKernelGGL((fa2::fwd_kernel<T, 128, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
+    case 192: hipLaunchKernelGGL((fa2::fwd_kernel<T, 192, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fa2::fwd_kernel<T, 256, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
   }
 }
 
@@ -117,7 +121,7 @@ bool direct_ok(const fa2::Tensor4 &t) { return t.stride_seq < (int64_t(1) << 24)
 template <typename T>
 void launch_fwd(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
   dim3 block(64 * fa2::kFwdWaves);
-  if (p.vec && p.headdim == dp && dp != 96 && direct_ok(p.k) && direct_ok(p.v)) {
+  if (p.vec && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128) && direct_ok(p.k) && direct_ok(p.v)) {
     switch (dp) {
       case 32: hipLaunchKernelGGL((fa2::fwd_direct_kernel<T, 32, kFwdBlockKV>), grid, block, 0, s, p); break;
       case 64: hipLaunchKernelGGL((fa2::fwd_direct_kernel<T, 64, kFwdBlockKV>), grid, block, 0, s, p); break;
@@ -134,7 +138,7 @@ void launch_fwd(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
 template <typename T>
 void launch_dq(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
   dim3 block(64 * fa2::kDqWaves);
-  if (p.vec && p.headdim == dp && dp != 96 && direct_ok(p.k) && direct_ok(p.v)) {
+  if (p.vec && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128) && direct_ok(p.k) && direct_ok(p.v)) {
     switch (dp) {
       case 32: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 32, kDqBlockKV>), grid, block, 0, s, p); break;
       case 64: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 64, kDqBlockKV>), grid, block, 0, s, p); break;
@@ -146,14 +150,16 @@ void launch_dq(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
     case 32: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 32, kDqBlockKV>), grid, block, 0, s, p); break;
     case 64: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 64, kDqBlockKV>), grid, block, 0, s, p); break;
     case 96: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 96, kDqBlockKV>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 128, kDqBlockKV>), grid, block, 0, s, p); break;
+    case 128: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 128, kDqBlockKV>), grid, block, 0, s, p); break;
+    case 192: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 192, kDqBlockKV>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 256, kDqBlockKV>), grid, block, 0, s, p); break;
   }
 }
 
 template <typename T>
 void launch_dkdv(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
   dim3 block(64 * fa2::kDkvWaves);
-  if (p.vec && p.headdim == dp && dp != 96 && direct_ok(p.q) && direct_ok(p.d_o)) {
+  if (p.vec && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128) && direct_ok(p.q) && direct_ok(p.d_o)) {
     switch (dp) {
       case 32: hipLaunchKernelGGL((fa2::bwd_dkdv_direct_kernel<T, 32, kDkvBlockQ>), grid, block, 0, s, p); break;
       case 64: hipLaunchKernelGGL((fa2::bwd_dkdv_direct_kernel<T, 64, kDkvBlockQ>), grid, block, 0, s, p); break;
@@ -165,7 +171,9 @@ void launch_dkdv(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
     case 32: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 32, kDkvBlockQ>), grid, block, 0, s, p); break;
     case 64: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 64, kDkvBlockQ>), grid, block, 0, s, p); break;
     case 96: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 96, kDkvBlockQ>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 128, kDkvBlockQ>), grid, block, 0, s, p); break;
+    case 128: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 128, kDkvBlockQ>), grid, block, 0, s, p); break;
+    case 192: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 192, kDkvBlockQ>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 256, kDkvBlockQ>), grid, block, 0, s, p); break;
   }
 }
 

@@ -138,7 +138,7 @@ __device__ __forceinline__ void fwd_tile(const short *sk, const short *sv, const
 }
 
 template <typename T, int DP, int BKV, bool VEC>
-__global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_kernel(const FwdParams p) {
   using L = FwdLayout<DP, BKV>;
   constexpr int KS = DP / 16;    // k-steps of Q K^T
   constexpr int DB = DP / 32;    // 32-row blocks of O^T

@@ -36,7 +36,7 @@ extern "C" {
 #define FA2_ABI_VERSION 1
 
 /* Largest head dimension the kernels accept (the table's `max_headdim`). */
-#define FA2_MAX_HEADDIM 128
+#define FA2_MAX_HEADDIM 256
 
 typedef enum fa2_status {
   FA2_OK = 0,

@@ -53,10 +53,11 @@ def test_abi_version_and_table(capi):
         assert r["fwd_block_q"] == 32 * r["fwd_waves"]
         assert r["bwd_block_kv"] == 32 * r["bwd_waves"]
         assert r["dq_block_q"] == 32 * r["dq_waves"]
-    for d, want in ((1, 32), (32, 32), (33, 64), (48, 64), (64, 64), (96, 96), (100, 128), (128, 128)):
+    for d, want in ((1, 32), (32, 32), (33, 64), (48, 64), (64, 64), (96, 96), (100, 128), (128, 128),
+                    (129, 192), (192, 192), (193, 256), (256, 256)):
         idx = lib.fa2_pick_config(capi.FA2_DTYPE_BF16, d, 512, 512, 0)
         assert idx >= 0 and rows[idx]["headdim_padded"] == want
-    assert lib.fa2_pick_config(capi.FA2_DTYPE_BF16, 129, 512, 512, 0) == -4  # FA2_ERR_HEADDIM
+    assert lib.fa2_pick_config(capi.FA2_DTYPE_BF16, 257, 512, 512, 0) == -4  # FA2_ERR_HEADDIM
     assert lib.fa2_pick_config(7, 64, 512, 512, 0) == -3  # FA2_ERR_BAD_DTYPE
     info = capi.ConfigInfo()
     assert lib.fa2_config_get(99, ctypes.byref(info)) == 6  # FA2_ERR_BAD_CONFIG
@@ -80,7 +81,7 @@ def _fwd_args(capi, **over):
     (dict(batch=0), "FA2_ERR_BAD_SHAPE"),
     (dict(seqlen_k=-3), "FA2_ERR_BAD_SHAPE"),
     (dict(seqlen_q=300, seqlen_q_rounded=256), "FA2_ERR_BAD_SHAPE"),
-    (dict(headdim=136), "FA2_ERR_HEADDIM"),
+    (dict(headdim=264), "FA2_ERR_HEADDIM"),
     (dict(dtype=5), "FA2_ERR_BAD_DTYPE"),
     (dict(config=17), "FA2_ERR_BAD_CONFIG"),
     (dict(config=0, headdim=64), "FA2_ERR_BAD_CONFIG"),  # row 0 is built for headdim <= 32
@@ -193,8 +194,8 @@ def test_launcher_assertions_mirror_reference(fa2_module):
         fwd(q, torch.zeros(1, 2, 8, 32, dtype=torch.float16), q, None, *tail)  # k shape
     with pytest.raises(AssertionError):
         fwd(q, q, torch.zeros(1, 3, 8, 16, dtype=torch.float16), None, *tail)  # v shape
-    big = torch.zeros(1, 1, 4, 256, dtype=torch.float16)
-    with pytest.raises(AssertionError, match="Supports head dimensions only up to 128"):
+    big = torch.zeros(1, 1, 4, 264, dtype=torch.float16)
+    with pytest.raises(AssertionError, match="Supports head dimensions only up to 256"):
         fwd(big, big, big, None, *tail)
     with pytest.raises(AssertionError, match="must reside on CUDA device"):
         fwd(q, q, q, None, *tail)

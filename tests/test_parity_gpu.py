@@ -75,6 +75,10 @@ SMALL_CASES = [
     (1, 2, 77, 1, 64, torch.bfloat16, 1.0),
     (1, 4, 640, 640, 64, torch.float16, 3.0),     # peaky softmax
     (1, 2, 257, 257, 128, torch.float16, 1.0),
+    (1, 2, 200, 200, 160, torch.bfloat16, 1.0),   # head dims above 128: padded to 192 / 256
+    (1, 2, 333, 200, 192, torch.float16, 1.0),
+    (2, 2, 300, 300, 256, torch.bfloat16, 1.0),
+    (1, 1, 130, 130, 250, torch.float16, 1.0),    # above 128 and not a multiple of 8
 ]
 
 
@@ -358,6 +362,6 @@ def test_device_side_assertions(fa):
     q = torch.zeros(1, 2, 16, 64, device="cuda", dtype=torch.float16)
     with pytest.raises(AssertionError):
         fa.flash_attention_v2(q, torch.zeros(1, 2, 16, 32, device="cuda", dtype=torch.float16), q)
-    big = torch.zeros(1, 1, 8, 160, device="cuda", dtype=torch.float16)
+    big = torch.zeros(1, 1, 8, 264, device="cuda", dtype=torch.float16)
     with pytest.raises(AssertionError, match="Supports head dimensions only up to"):
         fa.flash_attention_v2(big, big, big)
