@@ -80,13 +80,17 @@ def _flash_attention_forward(
     seqlen_q_rounded = math.ceil(seqlen_q / max_headdim) * max_headdim
     lse = torch.empty((batch, nheads, seqlen_q_rounded), device=q.device, dtype=torch.float32)
 
+    # The kernels take a positive scale.  A negative one (the reference passes any non-zero value
+    # through) is folded into the sign of Q, which is exact: (-Q) K^T * |s| == Q K^T * s.
+    q_in, kernel_scale = (q, softmax_scale) if softmax_scale > 0 else (-q, -softmax_scale)
+
     lib = _capi.load()
     with torch.cuda.device(q.device):
         status = lib.fa2_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), lse.data_ptr(),
+            q_in.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), lse.data_ptr(),
             batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded,
-            *_strides3(q), *_strides3(k), *_strides3(v), *_strides3(output),
-            softmax_scale, _COMPUTE_DTYPES[q.dtype], _capi.FA2_CONFIG_AUTO, _stream_handle(),
+            *_strides3(q_in), *_strides3(k), *_strides3(v), *_strides3(output),
+            kernel_scale, _COMPUTE_DTYPES[q.dtype], _capi.FA2_CONFIG_AUTO, _stream_handle(),
         )
     _capi.check(status, "fa2_fwd")
     return output, lse, softmax_scale  # softmax_scale could have been updated
@@ -133,6 +137,12 @@ def _flash_attention_backward(
     deterministic = 1 if kernels_config.deterministic else 0
     dtype = _COMPUTE_DTYPES[q.dtype]
 
+    # Negative scale: run on -Q with |scale| (see the forward launcher); dK and dV are unchanged
+    # and dQ comes out with the opposite sign.
+    negated = softmax_scale < 0
+    if negated:
+        q, softmax_scale = -q, -softmax_scale
+
     lib = _capi.load()
     with torch.cuda.device(q.device):
         stream = _stream_handle()
@@ -157,6 +167,8 @@ def _flash_attention_backward(
             softmax_scale, dtype, deterministic, _capi.FA2_CONFIG_AUTO, stream,
         )
         _capi.check(status, "fa2_bwd")
+    if negated:
+        dq.neg_()
 
 
 def _compute_dtype(dtype: torch.dtype) -> torch.dtype:

@@ -358,6 +358,16 @@ def test_zero_scale_means_default_and_explicit_scale_is_used(fa):
     _assert_close("o (scale 0.5)", c, oracle.naive_causal_attention(q, k, v, 0.5))
 
 
+def test_negative_scale(fa):
+    """The reference passes any non-zero scale to its kernels (flash_attention_2.py:94); a negative
+    one turns the softmax towards the smallest scores."""
+    q, k, v, d_o = _seeded((1, 2, 200, 64), (1, 2, 200, 64), torch.float16)
+    want = oracle.naive_backward(q, k, v, d_o, -0.2, torch.float32)
+    got = _run(fa, q, k, v, d_o, -0.2, True)
+    for name, g, w in zip(("o", "dq", "dk", "dv"), got, want):
+        _assert_close(name, g, w)
+
+
 def test_device_side_assertions(fa):
     q = torch.zeros(1, 2, 16, 64, device="cuda", dtype=torch.float16)
     with pytest.raises(AssertionError):
