@@ -114,7 +114,17 @@ def _kernel_legs(capi, w, q, k, v, d_o, iters: int):
                                *s3(dq), *s3(dk), *s3(dv), scale, dtype, det,
                                capi.FA2_CONFIG_AUTO, stream), "fa2_bwd")
 
+    def bwd_fused():
+        capi.check(lib.fa2_bwd_fused(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(),
+                                     lse.data_ptr(), delta.data_ptr(), ws.data_ptr(),
+                                     dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                     b, h, n, n, d, n_r, *s3(q), *s3(k), *s3(v), *s3(o), *s3(d_o),
+                                     *s3(dq), *s3(dk), *s3(dv), scale, dtype, 0,
+                                     capi.FA2_CONFIG_AUTO, stream), "fa2_bwd_fused")
+
     legs = {
+        # What autograd runs: dQ (forming delta on the way) then dK/dV, no preprocess launch.
+        "bwd_fused": bwd_fused,
         "bwd_deterministic": lambda: bwd(1),
         "bwd_sequence_parallel": lambda: bwd(0),
         # One kernel each: NULL outputs switch the other kernel off.
@@ -240,7 +250,7 @@ def main() -> int:
                 "avg_launch_ms": leg_ms[name]}
 
     roofline = mfma_roofline(dominant)
-    bwd_leg = "bwd_deterministic" if det else "bwd_sequence_parallel"
+    bwd_leg = "bwd_fused"
     bwd_tflops = w.bwd_flops / (leg_ms[bwd_leg] * 1e-3) / 1e12
     pre_bytes = 2.0 * w.batch * w.nheads * w.seqlen * w.headdim * 2 + w.batch * w.nheads * w.seqlen * 4
     pre_roofline = {

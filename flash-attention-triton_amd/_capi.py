@@ -47,6 +47,7 @@ SIGNATURES = {
     "fa2_bwd_preprocess": (_i, [_p] * 3 + [_i] * 5 + [_i64] * 6 + [_i, _p]),
     "fa2_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 7),
     "fa2_bwd": (_i, [_p] * 10 + [_i] * 6 + [_i64] * 21 + [_f, _i, _i, _i, _p]),
+    "fa2_bwd_fused": (_i, [_p] * 11 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p]),
 }
 
 _lib = None

@@ -29,6 +29,8 @@ namespace fa2 {
 
 struct BwdParams {
   Tensor4 q, k, v, d_o, dq, dk, dv;
+  Tensor4 o;         // only read by the dQ kernel when it also forms delta
+  float *delta_out;  // where that kernel writes delta (the same buffer `delta` points to)
   const float *lse;
   const float *delta;
   int batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded;
@@ -482,7 +484,10 @@ struct DqDirectLayout {
       (2 * STAGE_ELEMS > PATCH_ELEMS) ? 2 * STAGE_ELEMS : PATCH_ELEMS;
 };
 
-template <typename T, int DP, int BKV>
+// With FUSE_DELTA the kernel also computes delta = rowsum(O * dO) for its query rows (it holds
+// the dO rows anyway), uses it and writes it out for the dK/dV kernel, which then has to be
+// launched after this one; the separate preprocess launch disappears.
+template <typename T, int DP, int BKV, bool FUSE_DELTA>
 __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const BwdParams p) {
   using L = DqDirectLayout<DP, BKV>;
   constexpr int KS = DP / 16, DB = DP / 32;
@@ -546,8 +551,23 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
       qf[ks] = load_chunk(qp, 16 * ks + 8 * h, DP, ok, true);
       gf[ks] = load_chunk(gp, 16 * ks + 8 * h, DP, ok, true);
     }
-    if (ok) {
-      lse2 = p.lse[(int64_t)bh * p.seqlen_q_rounded + row] * kLog2e;
+    if (ok) lse2 = p.lse[(int64_t)bh * p.seqlen_q_rounded + row] * kLog2e;
+    if (FUSE_DELTA) {
+      const short *op = (const short *)p.o.ptr + b * p.o.stride_batch + hd * p.o.stride_head +
+                        (int64_t)row * p.o.stride_seq;
+      float part = 0.f;  // this lane's half of the row: columns 16 ks + 8 h + j
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        const s16x8 of = load_chunk(op, 16 * ks + 8 * h, DP, ok, true);
+#pragma unroll
+        for (int j = 0; j < 8; j++) part += Elem<T>::to_float(of[j]) * Elem<T>::to_float(gf[ks][j]);
+      }
+      delta = sum_over_halves(part);  // 0 for rows beyond the sequence (loads return zeros)
+      float *dout = p.delta_out + (int64_t)bh * p.seqlen_q_rounded;
+      if (h == 0 && ok) dout[row] = delta;
+      if (qt == p.n_tiles - 1)  // rows [seqlen_q, seqlen_q_rounded) are defined to be zero
+        for (int r = p.seqlen_q + tid; r < p.seqlen_q_rounded; r += 64 * kDqWaves) dout[r] = 0.f;
+    } else if (ok) {
       delta = p.delta[(int64_t)bh * p.seqlen_q_rounded + row];
     }
   }
@@ -744,20 +764,14 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(cons
       vf[ks] = load_chunk(vp, 16 * ks + 8 * h, DP, ok, true);
     }
   }
-  {
-    float l3[L::STAGES], d3[L::STAGES];
+  // Statistics of the first three tiles: loaded now, written to LDS just before the first
+  // barrier (the write has to wait for every load above, and the set-up below should not).
+  float l3[L::STAGES], d3[L::STAGES];
 #pragma unroll
-    for (int t = 0; t < L::STAGES; t++) {
-      load_stats(t);  // rows beyond the sequence (and tiles beyond the last) read as 0
-      l3[t] = lse_reg;
-      d3[t] = delta_reg;
-    }
-#pragma unroll
-    for (int t = 0; t < L::STAGES; t++) {
-      lse_reg = l3[t];
-      delta_reg = d3[t];
-      store_stats(t);
-    }
+  for (int t = 0; t < L::STAGES; t++) {
+    load_stats(t);  // rows beyond the sequence (and tiles beyond the last) read as 0
+    l3[t] = lse_reg;
+    d3[t] = delta_reg;
   }
 
   // Swizzled fragment addresses (32-bit LDS pointers) into the current tile's stage; the dO tile
@@ -793,6 +807,12 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(cons
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const int kvcol = kv0w + c;
 
+#pragma unroll
+  for (int t = 0; t < L::STAGES; t++) {
+    lse_reg = l3[t];
+    delta_reg = d3[t];
+    store_stats(t);
+  }
   bwd_wait_vmem_all();
   __syncthreads();
 

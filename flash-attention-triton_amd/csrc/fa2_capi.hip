@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -135,15 +136,25 @@ void launch_fwd(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
     launch_fwd_v<T, false>(dp, p, grid, s);
 }
 
+bool dq_direct_ok(int dp, const fa2::BwdParams &p) {
+  return p.vec && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128) && direct_ok(p.k) && direct_ok(p.v);
+}
+
+template <typename T, bool FUSE_DELTA>
+void launch_dq_direct(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
+  dim3 block(64 * fa2::kDqWaves);
+  switch (dp) {
+    case 32: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 32, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
+    case 64: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 64, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 128, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
+  }
+}
+
 template <typename T>
 void launch_dq(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
   dim3 block(64 * fa2::kDqWaves);
-  if (p.vec && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128) && direct_ok(p.k) && direct_ok(p.v)) {
-    switch (dp) {
-      case 32: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 32, kDqBlockKV>), grid, block, 0, s, p); break;
-      case 64: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 64, kDqBlockKV>), grid, block, 0, s, p); break;
-      default: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 128, kDqBlockKV>), grid, block, 0, s, p); break;
-    }
+  if (dq_direct_ok(dp, p)) {
+    launch_dq_direct<T, false>(dp, p, grid, s);
     return;
   }
   switch (dp) {
@@ -306,35 +317,39 @@ size_t fa2_bwd_workspace_bytes(int batch, int nheads, int seqlen_q, int seqlen_k
   return 0;
 }
 
-int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const float *lse,
-            const float *delta, void *workspace, void *dq, void *dk, void *dv, int batch,
-            int nheads, int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded, int64_t q_sb,
-            int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb,
-            int64_t v_sh, int64_t v_ss, int64_t do_sb, int64_t do_sh, int64_t do_ss, int64_t dq_sb,
-            int64_t dq_sh, int64_t dq_ss, int64_t dk_sb, int64_t dk_sh, int64_t dk_ss,
-            int64_t dv_sb, int64_t dv_sh, int64_t dv_ss, float softmax_scale, int dtype,
-            int deterministic, int config_id, void *stream) {
-  (void)workspace;
-  (void)deterministic;
+namespace {
+
+// Shared by fa2_bwd and fa2_bwd_fused.  With `o` given, delta is an output: it is formed by the dQ
+// kernel when the fast dQ kernel applies (and the dK/dV kernel then runs second), otherwise by the
+// preprocess kernel launched from here.
+int bwd_impl(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+             const float *lse, float *delta, void *dq, void *dk, void *dv, int batch, int nheads,
+             int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded, const int64_t *st,
+             const int64_t *o_st, float softmax_scale, int dtype, int config_id, void *stream) {
   int rc = check_common(batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded, dtype);
   if (rc) return rc;
+  const bool fused = o != nullptr;
   fa2::BwdParams p;
-  p.q = tensor(q, q_sb, q_sh, q_ss);
-  p.k = tensor(k, k_sb, k_sh, k_ss);
-  p.v = tensor(v, v_sb, v_sh, v_ss);
-  p.d_o = tensor(d_o, do_sb, do_sh, do_ss);
-  p.dq = tensor(dq, dq_sb, dq_sh, dq_ss);
-  p.dk = tensor(dk, dk_sb, dk_sh, dk_ss);
-  p.dv = tensor(dv, dv_sb, dv_sh, dv_ss);
+  p.q = tensor(q, st[0], st[1], st[2]);
+  p.k = tensor(k, st[3], st[4], st[5]);
+  p.v = tensor(v, st[6], st[7], st[8]);
+  p.d_o = tensor(d_o, st[9], st[10], st[11]);
+  p.dq = tensor(dq, st[12], st[13], st[14]);
+  p.dk = tensor(dk, st[15], st[16], st[17]);
+  p.dv = tensor(dv, st[18], st[19], st[20]);
+  p.o = fused ? tensor(o, o_st[0], o_st[1], o_st[2]) : fa2::Tensor4{nullptr, 0, 0, 0};
   // A caller that needs only part of the gradient passes NULL for the rest: dq == NULL skips the
   // dQ kernel, dk == dv == NULL skips the dK/dV kernel.  dk and dv come from one kernel, so they
   // are given or omitted together.
   const bool want_dq = dq != nullptr;
   const bool want_dkdv = dk != nullptr || dv != nullptr;
   if (!want_dq && !want_dkdv) return fail(FA2_ERR_NULL_POINTER, "dq, dk and dv are all NULL");
+  if (fused && !(want_dq && want_dkdv))
+    return fail(FA2_ERR_NULL_POINTER, "fa2_bwd_fused computes all of dq, dk and dv: none may be NULL");
   if ((rc = check_tensor("q", p.q)) || (rc = check_tensor("k", p.k)) ||
       (rc = check_tensor("v", p.v)) || (rc = check_tensor("d_o", p.d_o)))
     return rc;
+  if (fused && (rc = check_tensor("o", p.o))) return rc;
   if (want_dq && (rc = check_tensor("dq", p.dq))) return rc;
   if (want_dkdv && ((rc = check_tensor("dk", p.dk)) || (rc = check_tensor("dv", p.dv)))) return rc;
   if (lse == nullptr) return fail(FA2_ERR_NULL_POINTER, "lse is NULL");
@@ -346,6 +361,7 @@ int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const 
 
   p.lse = lse;
   p.delta = delta;
+  p.delta_out = delta;
   p.batch = batch;
   p.nheads = nheads;
   p.seqlen_q = seqlen_q;
@@ -362,24 +378,40 @@ int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const 
   const int dp = kTable[cfg].headdim_padded;
   const int64_t bh = (int64_t)batch * nheads;
 
-  if (want_dkdv) {  // dK, dV
-    fa2::BwdParams pk = p;
-    pk.n_tiles = (seqlen_k + fa2::kDkvBlockKV - 1) / fa2::kDkvBlockKV;
-    const int64_t nwg = pk.n_tiles * bh;
-    if (nwg > 0x7fffffff) return fail(FA2_ERR_TOO_LARGE, "grid of %lld workgroups too large", (long long)nwg);
-    dim3 grid((unsigned)nwg);
+  fa2::BwdParams pk = p, pq = p;
+  pk.n_tiles = (seqlen_k + fa2::kDkvBlockKV - 1) / fa2::kDkvBlockKV;
+  pq.n_tiles = (seqlen_q + fa2::kDqBlockQ - 1) / fa2::kDqBlockQ;
+  const int64_t nwg_k = pk.n_tiles * bh, nwg_q = pq.n_tiles * bh;
+  if (nwg_k > 0x7fffffff || nwg_q > 0x7fffffff)
+    return fail(FA2_ERR_TOO_LARGE, "grid of %lld workgroups too large", (long long)std::max(nwg_k, nwg_q));
+
+  auto run_dkdv = [&]() {
+    dim3 grid((unsigned)nwg_k);
     if (dtype == FA2_DTYPE_BF16)
       launch_dkdv<__bf16>(dp, pk, grid, s);
     else
       launch_dkdv<_Float16>(dp, pk, grid, s);
-    if ((rc = launch_status("fa2_bwd dK/dV launch"))) return rc;
+    return launch_status("fa2_bwd dK/dV launch");
+  };
+
+  if (fused && dq_direct_ok(dp, pq) && vec_ok(p.o, headdim)) {
+    // dQ first: it writes delta, which the dK/dV kernel reads.
+    dim3 grid((unsigned)nwg_q);
+    if (dtype == FA2_DTYPE_BF16)
+      launch_dq_direct<__bf16, true>(dp, pq, grid, s);
+    else
+      launch_dq_direct<_Float16, true>(dp, pq, grid, s);
+    if ((rc = launch_status("fa2_bwd_fused dQ launch"))) return rc;
+    return run_dkdv();
   }
-  if (want_dq) {  // dQ
-    fa2::BwdParams pq = p;
-    pq.n_tiles = (seqlen_q + fa2::kDqBlockQ - 1) / fa2::kDqBlockQ;
-    const int64_t nwg = pq.n_tiles * bh;
-    if (nwg > 0x7fffffff) return fail(FA2_ERR_TOO_LARGE, "grid of %lld workgroups too large", (long long)nwg);
-    dim3 grid((unsigned)nwg);
+  if (fused) {
+    rc = fa2_bwd_preprocess(o, d_o, delta, batch, nheads, seqlen_q, headdim, seqlen_q_rounded, o_st[0],
+                            o_st[1], o_st[2], st[9], st[10], st[11], dtype, stream);
+    if (rc) return rc;
+  }
+  if (want_dkdv && (rc = run_dkdv())) return rc;
+  if (want_dq) {
+    dim3 grid((unsigned)nwg_q);
     if (dtype == FA2_DTYPE_BF16)
       launch_dq<__bf16>(dp, pq, grid, s);
     else
@@ -387,6 +419,44 @@ int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const 
     if ((rc = launch_status("fa2_bwd dQ launch"))) return rc;
   }
   return FA2_OK;
+}
+
+}  // namespace
+
+int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const float *lse,
+            const float *delta, void *workspace, void *dq, void *dk, void *dv, int batch,
+            int nheads, int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded, int64_t q_sb,
+            int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb,
+            int64_t v_sh, int64_t v_ss, int64_t do_sb, int64_t do_sh, int64_t do_ss, int64_t dq_sb,
+            int64_t dq_sh, int64_t dq_ss, int64_t dk_sb, int64_t dk_sh, int64_t dk_ss,
+            int64_t dv_sb, int64_t dv_sh, int64_t dv_ss, float softmax_scale, int dtype,
+            int deterministic, int config_id, void *stream) {
+  (void)workspace;
+  (void)deterministic;  // both modes run the same atomic-free kernels
+  const int64_t st[21] = {q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, do_sb, do_sh,
+                          do_ss, dq_sb, dq_sh, dq_ss, dk_sb, dk_sh, dk_ss, dv_sb, dv_sh, dv_ss};
+  return bwd_impl(q, k, v, nullptr, d_o, lse, const_cast<float *>(delta), dq, dk, dv, batch, nheads,
+                  seqlen_q, seqlen_k, headdim, seqlen_q_rounded, st, nullptr, softmax_scale, dtype,
+                  config_id, stream);
+}
+
+int fa2_bwd_fused(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                  const float *lse, float *delta, void *workspace, void *dq, void *dk, void *dv,
+                  int batch, int nheads, int seqlen_q, int seqlen_k, int headdim,
+                  int seqlen_q_rounded, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb,
+                  int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int64_t o_sb,
+                  int64_t o_sh, int64_t o_ss, int64_t do_sb, int64_t do_sh, int64_t do_ss,
+                  int64_t dq_sb, int64_t dq_sh, int64_t dq_ss, int64_t dk_sb, int64_t dk_sh,
+                  int64_t dk_ss, int64_t dv_sb, int64_t dv_sh, int64_t dv_ss, float softmax_scale,
+                  int dtype, int deterministic, int config_id, void *stream) {
+  (void)workspace;
+  (void)deterministic;
+  if (o == nullptr) return fail(FA2_ERR_NULL_POINTER, "o is NULL");
+  const int64_t st[21] = {q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, do_sb, do_sh,
+                          do_ss, dq_sb, dq_sh, dq_ss, dk_sb, dk_sh, dk_ss, dv_sb, dv_sh, dv_ss};
+  const int64_t o_st[3] = {o_sb, o_sh, o_ss};
+  return bwd_impl(q, k, v, o, d_o, lse, delta, dq, dk, dv, batch, nheads, seqlen_q, seqlen_k, headdim,
+                  seqlen_q_rounded, st, o_st, softmax_scale, dtype, config_id, stream);
 }
 
 #ifdef FA2_WG_STAMPS

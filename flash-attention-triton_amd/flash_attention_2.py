@@ -146,27 +146,21 @@ def _flash_attention_backward(
     lib = _capi.load()
     with torch.cuda.device(q.device):
         stream = _stream_handle()
-        status = lib.fa2_bwd_preprocess(
-            output.data_ptr(), d_output.data_ptr(), delta.data_ptr(),
-            batch, nheads, seqlen_q, headdim, seqlen_q_rounded,
-            *_strides3(output), *_strides3(d_output), dtype, stream,
-        )
-        _capi.check(status, "fa2_bwd_preprocess")
-
         ws_bytes = lib.fa2_bwd_workspace_bytes(batch, nheads, seqlen_q, seqlen_k, headdim,
                                                deterministic, _capi.FA2_CONFIG_AUTO)
         workspace = (torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None)
-        status = lib.fa2_bwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), d_output.data_ptr(),
+        # Both launches of the reference launcher (preprocess, then the main kernel) in one call.
+        status = lib.fa2_bwd_fused(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), d_output.data_ptr(),
             lse.data_ptr(), delta.data_ptr(),
             workspace.data_ptr() if workspace is not None else None,
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
             batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded,
-            *_strides3(q), *_strides3(k), *_strides3(v), *_strides3(d_output),
+            *_strides3(q), *_strides3(k), *_strides3(v), *_strides3(output), *_strides3(d_output),
             *_strides3(dq), *_strides3(dk), *_strides3(dv),
             softmax_scale, dtype, deterministic, _capi.FA2_CONFIG_AUTO, stream,
         )
-        _capi.check(status, "fa2_bwd")
+        _capi.check(status, "fa2_bwd_fused")
     if negated:
         dq.neg_()
 

@@ -160,6 +160,30 @@ int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o,
             int64_t dv_stride_batch, int64_t dv_stride_head, int64_t dv_stride_seq,
             float softmax_scale, int dtype, int deterministic, int config_id, void *stream);
 
+/*
+ * Whole backward in one call: replaces both launches of _flash_attention_backward
+ * (flash_attention_2.py:218-277), i.e. fa2_bwd_preprocess followed by fa2_bwd, and gives the same
+ * dq, dk, dv (delta may differ in its last bits: the row sums are taken in another order).
+ * `delta` is an output here: fp32 (batch, nheads, seqlen_q_rounded) scratch supplied by the caller,
+ * filled like fa2_bwd_preprocess fills it.  When the fast dQ kernel applies, that kernel forms
+ * delta from the O and dO rows it already holds and the dK/dV kernel runs after it, which saves
+ * one launch and one pass over O and dO; otherwise the three kernels run as in the two-call path.
+ * dq, dk and dv must all be given.
+ */
+int fa2_bwd_fused(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                  const float *lse, float *delta, void *workspace,
+                  void *dq, void *dk, void *dv,
+                  int batch, int nheads, int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded,
+                  int64_t q_stride_batch, int64_t q_stride_head, int64_t q_stride_seq,
+                  int64_t k_stride_batch, int64_t k_stride_head, int64_t k_stride_seq,
+                  int64_t v_stride_batch, int64_t v_stride_head, int64_t v_stride_seq,
+                  int64_t o_stride_batch, int64_t o_stride_head, int64_t o_stride_seq,
+                  int64_t do_stride_batch, int64_t do_stride_head, int64_t do_stride_seq,
+                  int64_t dq_stride_batch, int64_t dq_stride_head, int64_t dq_stride_seq,
+                  int64_t dk_stride_batch, int64_t dk_stride_head, int64_t dk_stride_seq,
+                  int64_t dv_stride_batch, int64_t dv_stride_head, int64_t dv_stride_seq,
+                  float softmax_scale, int dtype, int deterministic, int config_id, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
