@@ -3,7 +3,7 @@
 
 A step is one forward + backward pass of ``flash_attention_v2`` through the real
 ``torch.autograd`` path on one batch of synthetic input already resident in HBM.  The workload
-is BASELINE's headline configuration C3 (B=2, H=32, N=4096, D=128, bf16, causal) unless
+is the headline configuration C3 (B=2, H=32, N=4096, D=128, bf16, causal) unless
 ``--workload`` names another one.  One JSON line is printed; ``value`` is forward+backward
 TFLOP/s with the FlashAttention-2 FLOP convention (fwd = 4*B*H*N^2*D/2, bwd = 2.5 x fwd), and
 the forward-only figures and fractions of the dense bf16 MFMA peak are in the same line.

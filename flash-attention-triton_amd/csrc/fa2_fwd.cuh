@@ -291,9 +291,6 @@ struct FwdDirectLayout {
 // s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt fields left at their maxima).
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-// Scheduling-group masks of __builtin_amdgcn_sched_group_barrier.
-constexpr int kSgValu = 0x002, kSgMfma = 0x008, kSgDsRead = 0x100, kSgTrans = 0x400;
-
 
 template <typename T, int DP, int BKV>
 __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const FwdParams p) {
@@ -409,23 +406,6 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
 #pragma unroll
     for (int i = 1; i < 16; i++) m = fmaxf(m, s[i]);
     return max_over_halves(m);
-  };
-  // P = exp2(scale*S - scale*m) rounded to T, plus the row sums of the rounded values.
-  auto softmax_block = [&](const f32x16 &s, s16x8 (&pf)[2]) {
-    const float mc = m_ref * scale_log2;
-    f32x16 e;
-#pragma unroll
-    for (int i = 0; i < 16; i++) e[i] = fast_exp2(s[i] * scale_log2 - mc);
-    f32x8 lo = {e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]};
-    f32x8 hi = {e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]};
-    pf[0] = Elem<T>::pack8(lo);
-    pf[1] = Elem<T>::pack8(hi);
-#pragma unroll
-    for (int ks2 = 0; ks2 < 2; ks2++) {
-      const u32x4 w = __builtin_bit_cast(u32x4, pf[ks2]);
-#pragma unroll
-      for (int j = 0; j < 4; j++) l_run = Elem<T>::add_pair(w[j], l_run);
-    }
   };
   // Raise the reference maximum when some row overshoots it by more than the slack.
   auto maybe_rescale = [&](float mloc) {

@@ -228,7 +228,7 @@ def test_fused_backward_matches_two_call_path(fa2_module, capi, name):
     assert lib.fa2_status_string(rc).decode() == "FA2_ERR_NULL_POINTER"
 
 
-# ------------------------------------------------------------------------- BASELINE configurations at full size
+# ------------------------------------------------------------------------- the five benchmark configurations at full size
 def _workload_case(workloads, name):
     w = workloads.WORKLOADS[name]
     q, k, v, d_o = workloads.make_inputs(w, "cpu")
