@@ -670,7 +670,7 @@ struct DkvDirectLayout {
 };
 
 template <typename T, int DP, int BQ>
-__global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_direct_kernel(const BwdParams p) {
+__global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_direct_kernel(const BwdParams p) {
   using L = DkvDirectLayout<DP, BQ>;
   constexpr int KS = DP / 16, DB = DP / 32;
   constexpr int NTHREADS = 64 * kDkvWaves;
