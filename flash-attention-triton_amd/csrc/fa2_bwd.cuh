@@ -525,14 +525,15 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   const int n_full = min(q0w + 1, seqlen_k) / BLK;                   // leading blocks without mask
   const int n_inside = seqlen_k / BKV;
 
+  const unsigned lds_base = lds_u32(smem);  // LDS byte address of smem
   auto issue_tile = [&](int t) {
-    short *dst = smem + (t & 1) * L::STAGE_ELEMS;
+    const unsigned dst = lds_base + 2u * (unsigned)((t & 1) * L::STAGE_ELEMS);
     if (t < n_inside) {
       kload.issue(t * BKV, dst);
-      vload.issue(t * BKV, dst + L::TILE_ELEMS);
+      vload.issue(t * BKV, dst + 2u * L::TILE_ELEMS);
     } else {
       kload.issue_clamped(t * BKV, seqlen_k, dst);
-      vload.issue_clamped(t * BKV, seqlen_k, dst + L::TILE_ELEMS);
+      vload.issue_clamped(t * BKV, seqlen_k, dst + 2u * L::TILE_ELEMS);
     }
   };
   issue_tile(0);
@@ -715,15 +716,16 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   // Tiles that touch the diagonal of this key tile (their blocks need the causal mask).
   const int n_diag = min(n_tiles, (kv0 + kDkvBlockKV - q_begin + BQ - 1) / BQ);
 
+  const unsigned lds_base = lds_u32(smem);  // LDS byte address of smem
   auto issue_tile = [&](int t) {
-    short *dst = smem + (t % L::STAGES) * L::STAGE_ELEMS;
+    const unsigned dst = lds_base + 2u * (unsigned)((t % L::STAGES) * L::STAGE_ELEMS);
     const int row0 = q_begin + t * BQ;
     if (t < n_inside) {
       qload.issue(row0, dst);
-      gload.issue(row0, dst + L::TILE_ELEMS);
+      gload.issue(row0, dst + 2u * L::TILE_ELEMS);
     } else {
       qload.issue_clamped(row0, seqlen_q, dst);
-      gload.issue_clamped(row0, seqlen_q, dst + L::TILE_ELEMS);
+      gload.issue_clamped(row0, seqlen_q, dst + 2u * L::TILE_ELEMS);
     }
   };
   // lse*log2e and delta of a tile go through registers into the stage's statistics area (rows

@@ -252,22 +252,25 @@ __device__ __forceinline__ int swz_off(int r, int c) { return r * DP + ((c ^ swz
 // to wait for the load (the compiler cannot tell which LDS bytes the DMA writes), which would
 // serialise the prefetch.  The callers order these loads against LDS reads themselves with
 // `s_waitcnt vmcnt(0)` followed by a workgroup barrier.
-__device__ __forceinline__ void load_lds_16(const short *gsrc, short *lds_wave_base) {
-  const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
-      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base);
+// LDS destinations are passed around as 32-bit byte addresses (wave-uniform integers): converting
+// a generic pointer into an LDS address costs a null check and 64-bit arithmetic per load, an
+// integer add does not.  lds_u32(p) does the conversion once.
+__device__ __forceinline__ unsigned lds_u32(const short *p) {
+  return (unsigned)__builtin_amdgcn_readfirstlane(
+      (int)(unsigned)(uintptr_t)(__attribute__((address_space(3))) const void *)p);
+}
+__device__ __forceinline__ void load_lds_16(const short *gsrc, unsigned lds_wave_addr) {
   asm volatile(
       "s_mov_b32 m0, %1\n\t"
       "s_nop 0\n\t"
       "global_load_lds_dwordx4 %0, off"
       :
-      : "v"(gsrc), "s"(lds_addr)
+      : "v"(gsrc), "s"(lds_wave_addr)
       : "memory");
 }
 // Same with the address split into a wave-uniform base (SGPR pair) and a per-lane byte offset.
 __device__ __forceinline__ void load_lds_16(const short *uniform_base, unsigned lane_byte_offset,
-                                            short *lds_wave_base) {
-  const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
-      (unsigned)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base);
+                                            unsigned lds_wave_addr) {
   // State the uniformity the "s" constraints need (folds away when the value is already scalar).
   const uint64_t raw = (uint64_t)(uintptr_t)uniform_base;
   // (readfirstlane returns a signed int: go through unsigned so the low word is not sign-extended)
@@ -280,7 +283,7 @@ __device__ __forceinline__ void load_lds_16(const short *uniform_base, unsigned 
       "s_nop 0\n\t"
       "global_load_lds_dwordx4 %0, %1"
       :
-      : "v"(lane_byte_offset), "s"(uniform_base), "s"(lds_addr)
+      : "v"(lane_byte_offset), "s"(uniform_base), "s"(lds_wave_addr)
       : "memory");
 }
 
@@ -313,21 +316,21 @@ struct TileLoader {
     voff = 2u * (unsigned)(row_in * (int)stride + chunk * 8);
   }
 
-  // Rows [row0, row0 + ROWS), all inside the matrix -> tile at `lds`.
-  __device__ __forceinline__ void issue(int row0, short *lds) const {
+  // Rows [row0, row0 + ROWS), all inside the matrix -> tile at LDS byte address `lds`.
+  __device__ __forceinline__ void issue(int row0, unsigned lds) const {
     const short *tile = base + (int64_t)row0 * stride;
 #pragma unroll
     for (int i = 0; i < LOADS; i++)
-      load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (i * NW + wave) * 512);
+      load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (unsigned)(i * NW + wave) * 1024u);
   }
 
   // Same, but rows at or beyond `nrows` are taken from row nrows - 1 (finite values that the
   // caller masks).
-  __device__ __forceinline__ void issue_clamped(int row0, int nrows, short *lds) const {
+  __device__ __forceinline__ void issue_clamped(int row0, int nrows, unsigned lds) const {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
       const int r = min(row0 + i * NW * RPL + row_in, nrows - 1);
-      load_lds_16(base + (int64_t)r * stride + chunk * 8, lds + (i * NW + wave) * 512);
+      load_lds_16(base + (int64_t)r * stride + chunk * 8, lds + (unsigned)(i * NW + wave) * 1024u);
     }
   }
 };

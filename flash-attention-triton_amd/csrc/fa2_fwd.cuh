@@ -335,12 +335,13 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   const int n_full = min(q0w + 1, seqlen_k) / BLK;
   const int n_inside = seqlen_k / BKV;  // tiles whose every row exists
 
+  const unsigned lds_base = lds_u32(smem);  // LDS byte address of smem
   auto issue_k = [&](int t) {
-    short *dst = smem + L::K_BASE + (t % L::K_STAGES) * L::TILE_ELEMS;
+    const unsigned dst = lds_base + 2u * (unsigned)(L::K_BASE + (t % L::K_STAGES) * L::TILE_ELEMS);
     if (t < n_inside) kload.issue(t * BKV, dst); else kload.issue_clamped(t * BKV, seqlen_k, dst);
   };
   auto issue_v = [&](int t) {
-    short *dst = smem + L::V_BASE + (t % L::V_STAGES) * L::TILE_ELEMS;
+    const unsigned dst = lds_base + 2u * (unsigned)(L::V_BASE + (t % L::V_STAGES) * L::TILE_ELEMS);
     if (t < n_inside) vload.issue(t * BKV, dst); else vload.issue_clamped(t * BKV, seqlen_k, dst);
   };
   issue_k(0);
