@@ -111,8 +111,9 @@ __global__ __launch_bounds__(64 * kDqWaves, (DP <= 96 ? 2 : 1)) void bwd_dq_kern
   const int i16 = lane & 15, g2 = (lane >> 4) & 1;
 
   const int BH = p.batch * p.nheads;
-  const int bh = blockIdx.x % BH;
-  const int qt = p.n_tiles - 1 - blockIdx.x / BH;
+  int bh, rank;
+  map_workgroup(blockIdx.x, BH, p.n_tiles, bh, rank);
+  const int qt = p.n_tiles - 1 - rank;  // the last query tile sees the most keys
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int q0 = qt * kDqBlockQ;
   const int q0w = q0 + 32 * wave;
@@ -296,8 +297,8 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdPa
 
   // Key tile 0 has the longest query range: issue tiles in ascending order (heaviest first).
   const int BH = p.batch * p.nheads;
-  const int bh = blockIdx.x % BH;
-  const int kt = blockIdx.x / BH;
+  int bh, kt;  // key tile 0 has the longest query range: rank == key tile
+  map_workgroup(blockIdx.x, BH, p.n_tiles, bh, kt);
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int kv0 = kt * kDkvBlockKV;
   const int kv0w = kv0 + 32 * wave;
@@ -503,8 +504,9 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   const int i16 = lane & 15, g2 = (lane >> 4) & 1;
 
   const int BH = p.batch * p.nheads;
-  const int bh = blockIdx.x % BH;
-  const int qt = p.n_tiles - 1 - blockIdx.x / BH;
+  int bh, rank;
+  map_workgroup(blockIdx.x, BH, p.n_tiles, bh, rank);
+  const int qt = p.n_tiles - 1 - rank;  // the last query tile sees the most keys
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int q0 = qt * kDqBlockQ;
   const int q0w = q0 + 32 * wave;
@@ -690,8 +692,8 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 
   // Key tile 0 has the longest query range: issue tiles in ascending order (heaviest first).
   const int BH = p.batch * p.nheads;
-  const int bh = blockIdx.x % BH;
-  const int kt = blockIdx.x / BH;
+  int bh, kt;  // key tile 0 has the longest query range: rank == key tile
+  map_workgroup(blockIdx.x, BH, p.n_tiles, bh, kt);
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int kv0 = kt * kDkvBlockKV;
   const int kv0w = kv0 + 32 * wave;

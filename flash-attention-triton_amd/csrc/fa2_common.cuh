@@ -211,6 +211,25 @@ __device__ __forceinline__ void store_transposed_acc(const f32x16 (&acc)[DP / 32
   }
 }
 
+// Workgroup index -> (batch*head, tile rank); rank 0 is the heaviest tile of a head.
+//
+// Heads are taken 64 at a time: all tiles of a group of 64 heads, heaviest first, before the next
+// group starts.  The tiles of one head re-read the same K/V (or Q/dO) rows, so they should run
+// close together in time; with the heads merely round-robin over the whole grid, a problem with
+// thousands of (batch, head) pairs would have as many different heads in flight as the chip has
+// workgroup slots, nothing would be shared in L2 and every tile would stream its operand from HBM.
+// Workgroups go to the 8 XCDs round-robin and 64 is a multiple of 8, so a head also stays on one
+// XCD (one L2).  Up to 64 heads the order is simply head = i % heads, rank = i / heads.
+constexpr int kHeadGroup = 64;
+__device__ __forceinline__ void map_workgroup(int i, int heads, int tiles_per_head, int &bh, int &rank) {
+  const int per_group = kHeadGroup * tiles_per_head;
+  const int g = i / per_group;
+  const int r = i - g * per_group;
+  const int gsize = min(kHeadGroup, heads - g * kHeadGroup);  // the last group may be smaller
+  bh = g * kHeadGroup + r % gsize;
+  rank = r / gsize;
+}
+
 #ifdef FA2_WG_STAMPS
 // Debug build only: wall-clock (100 MHz) stamps per workgroup: start, loop start, loop end, end.
 __device__ long long fa2_wg_stamps[8192][4];

@@ -12,8 +12,9 @@
 //  * The accumulator is O^T = V^T P^T.  P^T leaves the first MFMA in exactly the register layout
 //    the second MFMA wants for its B operand, so probabilities never touch LDS.  V^T fragments are
 //    read from the row-major V tile with the transposing LDS read.
-//  * K and V tiles are double-buffered in LDS; the next tile's global loads are in flight while
-//    the current tile is being multiplied.
+//  * K and V tiles are staged in LDS (two stages each in the generic kernel, three K stages and
+//    two V stages in the fast one); the next tiles' global loads are in flight while the current
+//    tile is being multiplied.
 //  * Unlike the reference (mask applied to every tile, lines 139-147) the mask is evaluated only
 //    on tiles that touch the diagonal or the end of the key sequence, and sub-blocks entirely
 //    above the diagonal are skipped.
@@ -158,8 +159,9 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_kerne
   // taking the head from id % BH keeps every tile of one head on one XCD's L2 when BH % 8 == 0;
   // query tiles are issued heaviest (longest key range) first.
   const int BH = p.batch * p.nheads;
-  const int bh = blockIdx.x % BH;
-  const int qt = p.n_qtiles - 1 - blockIdx.x / BH;
+  int bh, rank;
+  map_workgroup(blockIdx.x, BH, p.n_qtiles, bh, rank);
+  const int qt = p.n_qtiles - 1 - rank;  // the last query tile sees the most keys
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int q0 = qt * kFwdBlockQ;
   const int q0w = q0 + 32 * wave;
@@ -311,8 +313,9 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   const int i16 = lane & 15, g2 = (lane >> 4) & 1;
 
   const int BH = p.batch * p.nheads;
-  const int bh = blockIdx.x % BH;
-  const int qt = p.n_qtiles - 1 - blockIdx.x / BH;
+  int bh, rank;
+  map_workgroup(blockIdx.x, BH, p.n_qtiles, bh, rank);
+  const int qt = p.n_qtiles - 1 - rank;  // the last query tile sees the most keys
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int q0 = qt * kFwdBlockQ;
   const int q0w = q0 + 32 * wave;
