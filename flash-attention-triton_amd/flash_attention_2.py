@@ -42,6 +42,26 @@ def _stream_handle() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+class _NoGuard:
+    """Stands in for torch.cuda.device(...) when the tensors already live on the current device
+    (the usual case): entering a device guard costs several microseconds per launch."""
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _device_guard(device: torch.device):
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
 def _flash_attention_forward(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -85,7 +105,7 @@ def _flash_attention_forward(
     q_in, kernel_scale = (q, softmax_scale) if softmax_scale > 0 else (-q, -softmax_scale)
 
     lib = _capi.load()
-    with torch.cuda.device(q.device):
+    with _device_guard(q.device):
         status = lib.fa2_fwd(
             q_in.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), lse.data_ptr(),
             batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded,
@@ -144,7 +164,7 @@ def _flash_attention_backward(
         q, softmax_scale = -q, -softmax_scale
 
     lib = _capi.load()
-    with torch.cuda.device(q.device):
+    with _device_guard(q.device):
         stream = _stream_handle()
         ws_bytes = lib.fa2_bwd_workspace_bytes(batch, nheads, seqlen_q, seqlen_k, headdim,
                                                deterministic, _capi.FA2_CONFIG_AUTO)
