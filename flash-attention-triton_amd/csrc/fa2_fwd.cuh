@@ -411,35 +411,25 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
     for (int i = 1; i < 16; i++) m = fmaxf(m, s[i]);
     return max_over_halves(m);
   };
-  // Raise the reference maximum when some row overshoots it by more than the slack.
-  auto maybe_rescale = [&](float mloc) {
-    const bool grow = (mloc - m_ref) * scale_log2 > kRescaleSlack;
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-      const float m_new = fmaxf(m_ref, mloc);
-      const float alpha = fast_exp2((m_ref - m_new) * scale_log2);
-      m_ref = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
-    }
-  };
-
   wait_vmem_all();
   __syncthreads();
 
-  // ---- prologue: S_0, its row maximum, ring <- K fragments of block 1 -------------------------
+  // ---- prologue: S_0, its row maximum, e_0 = exp2(scale*S_0 - scale*m), ring <- K fragments of
+  // block 1 ---------------------------------------------------------------------------------
   s16x8 ring[KS];
-  f32x16 sa, sb;
+  f32x16 sc;  // the score block in flight (S_{j+1} during step j)
+  f32x16 e;   // unnormalised probabilities of the block whose P V product comes next
   {
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) ring[ks] = k_frag(0, ks);
-    sa = zero;
+    sc = zero;
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) sa = Elem<T>::mfma(ring[ks], qf[ks], sa);
-    if (0 >= n_full) apply_mask(sa, 0);
-    m_ref = row_max(sa);  // finite: every query row sees key 0
+    for (int ks = 0; ks < KS; ks++) sc = Elem<T>::mfma(ring[ks], qf[ks], sc);
+    if (0 >= n_full) apply_mask(sc, 0);
+    m_ref = row_max(sc);  // finite: every query row sees key 0
+    const float mc = m_ref * scale_log2;
+#pragma unroll
+    for (int i = 0; i < 16; i++) e[i] = fast_exp2(sc[i] * scale_log2 - mc);
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) ring[ks] = k_frag(1, ks);
     // From here on kcur addresses K tile 1 (the tile after the current one).
@@ -447,45 +437,52 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
     for (int ks = 0; ks < KS; ks++) kcur[ks] += L::TILE_ELEMS;
   }
 
-  // One block step: scur holds S_j (maximum already accounted for), snxt receives S_{j+1}.
-  // HALF (= j & 1) selects the half-tile: V_j is half HALF of the current V tile and K_{j+2} is
-  // half HALF of the next K tile.
+  // One block step.  On entry e holds the probabilities of block j (formed against m_ref) and the
+  // ring the K fragments of block j+1.
+  //     X: S_{j+1}^T = K_{j+1} Q^T   beside   pack P_j, add its row sums        ring <- V_j^T
+  //     Y: O^T += V_j^T P_j^T        beside   max and exponentials of S_{j+1}   ring <- K_{j+2}
+  // The exponentials, which do not overlap with MFMAs of their own wave and are the most expensive
+  // vector instructions here, sit in the phase whose MFMAs need the fewest LDS reads, which evens
+  // out the two phases.  HALF (= j & 1) selects the half-tile: V_j is half HALF of the current V
+  // tile and K_{j+2} is half HALF of the next K tile.
   //
   // The step is hand-interleaved: each unit is one MFMA, the LDS reads that refill the ring slot
   // it just freed, and a few vector instructions; a scheduling fence after every unit keeps the
   // compiler from regrouping them (which would lengthen live ranges past the register file).
   // S_{j+1} and the K fragments of block j+2 are produced even when those blocks are not this
   // wave's (the values are then never used), so that there is a single code path.
-  auto step = [&](int j, auto half_tag, f32x16 &scur, f32x16 &snxt) {
+  //
+  // The new probabilities are formed against the maximum in use; if S_{j+1} turns out to exceed
+  // it by more than the slack (rare once the maximum has settled), the running state is rescaled
+  // after the step's MFMAs and the probabilities are formed again.
+  auto step = [&](int j, auto half_tag) {
     constexpr int HALF = decltype(half_tag)::value;
     if (j >= n_mine) return;
-    const float mc = m_ref * scale_log2;
     typedef unsigned u32x4v __attribute__((ext_vector_type(4)));
     u32x4v w[2];  // packed probabilities, two per word: w[0] = k-step 0, w[1] = k-step 1
-    snxt = zero;
+    sc = zero;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      snxt = Elem<T>::mfma(ring[ks], qf[ks], snxt);
+      sc = Elem<T>::mfma(ring[ks], qf[ks], sc);
       ring[ks] = v_frag(HALF, ks / DB, ks % DB);
 #pragma unroll
       for (int u = 0; u < 8 / KS; u++) {
         const int i = (8 / KS) * ks + u;  // probability pair (2i, 2i+1) of the 32 in the block
-        const float e0 = fast_exp2(scur[2 * i] * scale_log2 - mc);
-        const float e1 = fast_exp2(scur[2 * i + 1] * scale_log2 - mc);
-        w[i / 4][i % 4] = Elem<T>::pack2(e0, e1);
-        l_run += e0;
-        l_run += e1;
+        w[i / 4][i % 4] = Elem<T>::pack2(e[2 * i], e[2 * i + 1]);
+        l_run += e[2 * i];
+        l_run += e[2 * i + 1];
       }
-      // Pin the arithmetic to this unit: without a use here the optimiser sinks it past the
-      // branch below, next to the MFMAs that consume it.
+      // Pin the arithmetic to this unit: without a use here the optimiser sinks it next to the
+      // MFMAs that consume it.
       asm volatile("" : "+v"(l_run));
       if (ks == KS / 2 - 1) asm volatile("" : "+v"(w[0]));
       if (ks == KS - 1) asm volatile("" : "+v"(w[1]));
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (j + 1 >= n_full) apply_mask(snxt, (j + 1) * BLK);
+    if (j + 1 >= n_full) apply_mask(sc, (j + 1) * BLK);
     const s16x8 pf[2] = {__builtin_bit_cast(s16x8, w[0]), __builtin_bit_cast(s16x8, w[1])};
-    float mloc = fmaxf(snxt[0], snxt[1]);
+    const float mc = m_ref * scale_log2;
+    float mloc = fmaxf(sc[0], sc[1]);
 #pragma unroll
     for (int ks2 = 0; ks2 < 2; ks2++) {
 #pragma unroll
@@ -493,21 +490,40 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
         const int slot = ks2 * DB + db;
         oacc[db] = Elem<T>::mfma(ring[slot], pf[ks2], oacc[db]);
         ring[slot] = k_frag(HALF, slot);
-        if (slot >= 1 && 2 * slot + 1 < 16) mloc = fmaxf(fmaxf(mloc, snxt[2 * slot]), snxt[2 * slot + 1]);
+#pragma unroll
+        for (int u = 0; u < 16 / KS; u++) {
+          const int i = (16 / KS) * slot + u;
+          if (i >= 2) mloc = fmaxf(mloc, sc[i]);
+          e[i] = fast_exp2(sc[i] * scale_log2 - mc);
+        }
         asm volatile("" : "+v"(mloc));
+        asm volatile("" : "+v"(e));
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-#pragma unroll
-    for (int i = 2 * KS; i < 16; i++) mloc = fmaxf(mloc, snxt[i]);
     mloc = max_over_halves(mloc);
-    if (j + 1 < n_mine) maybe_rescale(mloc);
+    if (j + 1 < n_mine) {
+      const bool grow = (mloc - m_ref) * scale_log2 > kRescaleSlack;
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+        const float m_new = fmaxf(m_ref, mloc);
+        const float alpha = fast_exp2((m_ref - m_new) * scale_log2);
+        m_ref = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+        const float mc2 = m_new * scale_log2;
+#pragma unroll
+        for (int i = 0; i < 16; i++) e[i] = fast_exp2(sc[i] * scale_log2 - mc2);
+      }
+    }
   };
 
   FA2_STAMP(1);
   for (int t = 0; t < n_tiles; t++) {
-    step(2 * t, std::integral_constant<int, 0>{}, sa, sb);
-    step(2 * t + 1, std::integral_constant<int, 1>{}, sb, sa);
+    step(2 * t, std::integral_constant<int, 0>{});
+    step(2 * t + 1, std::integral_constant<int, 1>{});
     // Every wave is done with K_t and V_t; K_{t+2} and V_{t+1} (issued one tile ago) have landed.
     wait_vmem_all();
     __syncthreads();
