@@ -57,6 +57,8 @@ def _event_time_ms(fn, iters: int) -> list[float]:
     """Per-call GPU time of ``fn`` measured with HIP events on torch's current stream, which is
     the stream the library launches on."""
     times = []
+    for _ in range(3):  # untimed: first launches of a kernel run at clocks that have not settled
+        fn()
     for _ in range(iters):
         start = torch.cuda.Event(enable_timing=True)
         end = torch.cuda.Event(enable_timing=True)
@@ -165,8 +167,9 @@ def _cpu_baseline(w, workloads, heads: int):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50,
+                    help="untimed steps first; the GPU clocks need some tens of milliseconds of load to settle")
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--deterministic", action="store_true", help="time the deterministic backward in the step")
     ap.add_argument("--cpu-heads", type=int, default=64, help="(batch, head) slices in the CPU baseline sample")

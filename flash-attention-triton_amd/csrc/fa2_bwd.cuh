@@ -602,19 +602,40 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   bwd_wait_vmem_all();
   __syncthreads();
 
-  for (int t = 0; t < n_tiles; t++) {
+  // Tiles [1, n_spread) bring in their successor during their first block, one global->LDS load
+  // every other MFMA of the first two GEMMs: issued back to back by all waves after a barrier the
+  // loads queue up in the memory pipeline, and a wave whose load cannot issue cannot issue its
+  // MFMAs either.  The other tiles' successors (ragged tiles, and tile 1) are loaded at once.
+  constexpr int LOADS = TileLoader<DP, BKV, kDqWaves>::LOADS;
+  static_assert(KS >= 2 * LOADS, "the first two GEMMs have a slot for every load");
+  const int n_spread = min(n_tiles, n_inside) - 1;
+  auto tile = [&](int t, auto spread_tag) {
+    constexpr bool SPREAD = decltype(spread_tag)::value;
     const int soff = (t & 1) * L::STAGE_ELEMS;
+    const unsigned ldst = lds_base + 2u * (unsigned)(((t + 1) & 1) * L::STAGE_ELEMS);
+    // Load li of the 2 LOADS that make up K tile t+1 and V tile t+1.
+    auto spread_load = [&](int li) {
+      if (li < LOADS) kload.issue_one((t + 1) * BKV, ldst, li);
+      else if (li < 2 * LOADS) vload.issue_one((t + 1) * BKV, ldst + 2u * L::TILE_ELEMS, li - LOADS);
+    };
 #pragma unroll
     for (int mb = 0; mb < 2; mb++) {
       const int j = 2 * t + mb;
+      const bool spread_here = SPREAD && mb == 0;
       if (j < n_mine) {
         const int koff = soff + mb * BLK * DP;
         const int voff = koff + L::TILE_ELEMS;
         f32x16 s = zero, dp = zero;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) s = Elem<T>::mfma(lds_read_128(krow[ks] + koff), qf[ks], s);
+        for (int ks = 0; ks < KS; ks++) {
+          s = Elem<T>::mfma(lds_read_128(krow[ks] + koff), qf[ks], s);
+          if (spread_here && ks % 2 == 0) spread_load(ks / 2);
+        }
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) dp = Elem<T>::mfma(lds_read_128(krow[ks] + voff), gf[ks], dp);
+        for (int ks = 0; ks < KS; ks++) {
+          dp = Elem<T>::mfma(lds_read_128(krow[ks] + voff), gf[ks], dp);
+          if (spread_here && ks % 2 == 0) spread_load(KS / 2 + ks / 2);
+        }
         const bool need_mask = j >= n_full;
         f32x16 ds;
 #pragma unroll
@@ -639,13 +660,22 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
             dqacc[db] = Elem<T>::mfma(a, dsf[ks2], dqacc[db]);
           }
         }
+      } else if (spread_here) {  // not reached: skipped blocks lie in the last two tiles
+        issue_tile(t + 1);
       }
     }
-    // Everyone is done with stage t & 1; tile t+1 (issued one tile ago) has landed.
+    // Everyone is done with stage t & 1; tile t+1 (issued during this tile or before) has landed.
     bwd_wait_vmem_all();
     __syncthreads();
-    if (t + 2 < n_tiles) issue_tile(t + 2);
+    if (t + 2 < n_tiles && t + 1 >= n_spread) issue_tile(t + 2);
+  };
+  int t = 0;
+  if (n_tiles > 0) {  // tile 1 was loaded before the loop
+    tile(0, std::false_type{});
+    t = 1;
   }
+  for (; t < n_spread; t++) tile(t, std::true_type{});
+  for (; t < n_tiles; t++) tile(t, std::false_type{});
 
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(dqacc, p.scale, patch, DQ + (int64_t)q0w * p.dq.stride_seq,
@@ -827,9 +857,24 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   for (int ks = 0; ks < KS; ks++) ring[ks] = lds_read_128(qrow[ks]);
 
   // One 32-row query block.  HALF selects the half-tile; MASKED switches the causal/row masks on.
-  auto block = [&](int qb, auto half_tag, auto masked_tag) {
+  // With SPREAD the block also issues the global->LDS loads of tile `lt`, one every fourth unit:
+  // issued back to back by all waves after a barrier they queue up in the memory pipeline, and a
+  // wave whose load cannot issue cannot issue its MFMAs either.
+  auto block = [&](int qb, auto half_tag, auto masked_tag, auto spread_tag, int lt) {
     constexpr int HALF = decltype(half_tag)::value;
     constexpr bool MASKED = decltype(masked_tag)::value;
+    constexpr bool SPREAD = decltype(spread_tag)::value;
+    constexpr int LOADS = TileLoader<DP, BQ, kDkvWaves>::LOADS;
+    static_assert(4 * KS == 8 * LOADS, "one load every fourth unit covers both tiles");
+    const unsigned ldst = lds_base + 2u * (unsigned)((lt % L::STAGES) * L::STAGE_ELEMS);
+    const int lrow0 = q_begin + lt * BQ;
+    auto spread_load = [&](int unit) {  // unit: 0 .. 4 KS - 1 over the four GEMMs
+      if (SPREAD && unit % 4 == 0) {
+        const int li = unit / 4;
+        if (li < LOADS) qload.issue_one(lrow0, ldst, li);
+        else gload.issue_one(lrow0, ldst + 2u * L::TILE_ELEMS, li - LOADS);
+      }
+    };
     constexpr int QOFF = HALF * 32 * DP;          // Q rows of this block inside the tile
     constexpr int GOFF = QOFF + L::TILE_ELEMS;    // dO rows of this block
     typedef const __attribute__((address_space(3))) f32x4 *stat4_ptr;
@@ -840,6 +885,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       s = Elem<T>::mfma(ring[ks], kf[ks], s);
+      spread_load(ks);
       ring[ks] = lds_read_128(qrow[ks] + GOFF);
       constexpr int PER = (4 + KS - 1) / KS;  // row groups of four fetched per unit
 #pragma unroll
@@ -857,6 +903,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       dp = Elem<T>::mfma(ring[ks], vf[ks], dp);
+      spread_load(KS + ks);
       {
         s16x4 a0 = lds_read_tr(qlo[ks % DB] + GOFF + 16 * (ks / DB) * DP);
         s16x4 a1 = lds_read_tr(qhi[ks % DB] + GOFF + 16 * (ks / DB) * DP);
@@ -883,6 +930,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       dvacc[ks % DB] = Elem<T>::mfma(ring[ks], pf[ks / DB], dvacc[ks % DB]);
+      spread_load(2 * KS + ks);
       {
         s16x4 a0 = lds_read_tr(qlo[ks % DB] + QOFF + 16 * (ks / DB) * DP);
         s16x4 a1 = lds_read_tr(qhi[ks % DB] + QOFF + 16 * (ks / DB) * DP);
@@ -903,26 +951,30 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       dkacc[ks % DB] = Elem<T>::mfma(ring[ks], dsf[ks / DB], dkacc[ks % DB]);
+      spread_load(3 * KS + ks);
       ring[ks] = lds_read_128(qnext[ks] + (HALF == 0 ? 32 * DP : 0));
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  auto tile = [&](int t, auto masked_tag) {
+  // Tiles [spread_lo, spread_hi) bring in the tile two after them during their first block; the
+  // other tiles' successors are loaded at once after the barrier that frees their stage.
+  const int spread_lo = n_diag, spread_hi = n_inside - 2;
+  auto tile = [&](int t, auto masked_tag, auto spread_tag) {
     const int qt0 = q_begin + t * BQ;
     // qnext -> next tile's stage before the second block prefetches from it.
     const int d = ((t + 1) % L::STAGES == 0) ? -(L::STAGES - 1) * L::STAGE_ELEMS : L::STAGE_ELEMS;
-    block(qt0, std::integral_constant<int, 0>{}, masked_tag);
+    block(qt0, std::integral_constant<int, 0>{}, masked_tag, spread_tag, t + 2);
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qnext[ks] += d;
-    block(qt0 + 32, std::integral_constant<int, 1>{}, masked_tag);
-    // Tile t+3's statistics were loaded one tile ago; their stage was freed by the last barrier.
+    block(qt0 + 32, std::integral_constant<int, 1>{}, masked_tag, std::false_type{}, 0);
+    // Tile t+2's statistics were loaded one tile ago; their stage was freed by the last barrier.
     if (t >= 1 && t + 2 < n_tiles) store_stats(t + 2);
-    // Everyone is done with stage t % 3; tile t+2 (issued one tile ago) has landed.
+    // Everyone is done with stage t % 3; tile t+1 has landed, tile t+2 is in flight.
     bwd_wait_vmem_all();
     __syncthreads();
     if (t + 3 < n_tiles) {
-      issue_tile(t + 3);
+      if (t + 1 < spread_lo || t + 1 >= spread_hi) issue_tile(t + 3);
       load_stats(t + 3);
     }
 #pragma unroll
@@ -936,9 +988,10 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   };
 
   int t = 0;
-  for (; t < n_diag; t++) tile(t, std::true_type{});
-  for (; t < n_inside; t++) tile(t, std::false_type{});
-  for (; t < n_tiles; t++) tile(t, std::true_type{});
+  for (; t < n_diag; t++) tile(t, std::true_type{}, std::false_type{});
+  for (; t < spread_hi; t++) tile(t, std::false_type{}, std::true_type{});
+  for (; t < n_inside; t++) tile(t, std::false_type{}, std::false_type{});
+  for (; t < n_tiles; t++) tile(t, std::true_type{}, std::false_type{});
   FA2_STAMP(2);
 
   short *patch = smem + wave * 32 * (DP + 8);

@@ -343,6 +343,13 @@ struct TileLoader {
       load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (unsigned)(i * NW + wave) * 1024u);
   }
 
+  // Wave-load i (0 <= i < LOADS) of the same tile alone, for callers that spread a tile's loads
+  // between other work.
+  __device__ __forceinline__ void issue_one(int row0, unsigned lds, int i) const {
+    const short *tile = base + (int64_t)row0 * stride;
+    load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (unsigned)(i * NW + wave) * 1024u);
+  }
+
   // Same, but rows at or beyond `nrows` are taken from row nrows - 1 (finite values that the
   // caller masks).
   __device__ __forceinline__ void issue_clamped(int row0, int nrows, unsigned lds) const {

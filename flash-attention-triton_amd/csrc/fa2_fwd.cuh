@@ -347,10 +347,10 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
     const unsigned dst = lds_base + 2u * (unsigned)(L::V_BASE + (t % L::V_STAGES) * L::TILE_ELEMS);
     if (t < n_inside) vload.issue(t * BKV, dst); else vload.issue_clamped(t * BKV, seqlen_k, dst);
   };
+  // K_0, V_0 and K_1 are loaded here; after that tile t brings in K_{t+2} and V_{t+1}.
   issue_k(0);
   issue_v(0);
-  if (n_tiles > 1) { issue_k(1); issue_v(1); }
-  if (n_tiles > 2) issue_k(2);
+  if (n_tiles > 1) issue_k(1);
 
   // Q^T fragments (B operand of S^T = K Q^T): lane (c, h) holds Q[q0w + c][16 ks + 8 h + j].
   s16x8 qf[KS];
@@ -455,15 +455,32 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   // The new probabilities are formed against the maximum in use; if S_{j+1} turns out to exceed
   // it by more than the slack (rare once the maximum has settled), the running state is rescaled
   // after the step's MFMAs and the probabilities are formed again.
-  auto step = [&](int j, auto half_tag) {
+  //
+  // Tile loads (SPREAD): the global->LDS loads of K tile t+2 and V tile t+1 are issued one at a
+  // time between the units of tile t's first step.  Issued back to back by all waves at once they
+  // queue up in the memory pipeline, and a wave whose load cannot issue cannot issue its MFMAs
+  // either.
+  constexpr int LOAD_EVERY = KS / TileLoader<DP, BKV, kFwdWaves>::LOADS;
+  auto step = [&](int j, auto half_tag, auto spread_tag) {
     constexpr int HALF = decltype(half_tag)::value;
-    if (j >= n_mine) return;
+    constexpr bool SPREAD = decltype(spread_tag)::value;
+    if (j >= n_mine) {
+      if (SPREAD) {  // not reached: the skipped blocks lie in the last two tiles, which load nothing
+        issue_k(j / 2 + 2);
+        issue_v(j / 2 + 1);
+      }
+      return;
+    }
+    const int kt = j / 2 + 2, vt = j / 2 + 1;  // tiles loaded during this step (SPREAD)
+    const unsigned kdst = lds_base + 2u * (unsigned)(L::K_BASE + (kt % L::K_STAGES) * L::TILE_ELEMS);
+    const unsigned vdst = lds_base + 2u * (unsigned)(L::V_BASE + (vt % L::V_STAGES) * L::TILE_ELEMS);
     typedef unsigned u32x4v __attribute__((ext_vector_type(4)));
     u32x4v w[2];  // packed probabilities, two per word: w[0] = k-step 0, w[1] = k-step 1
     sc = zero;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       sc = Elem<T>::mfma(ring[ks], qf[ks], sc);
+      if (SPREAD && ks % LOAD_EVERY == 0) vload.issue_one(vt * BKV, vdst, ks / LOAD_EVERY);
       ring[ks] = v_frag(HALF, ks / DB, ks % DB);
 #pragma unroll
       for (int u = 0; u < 8 / KS; u++) {
@@ -489,6 +506,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
       for (int db = 0; db < DB; db++) {
         const int slot = ks2 * DB + db;
         oacc[db] = Elem<T>::mfma(ring[slot], pf[ks2], oacc[db]);
+        if (SPREAD && slot % LOAD_EVERY == 0) kload.issue_one(kt * BKV, kdst, slot / LOAD_EVERY);
         ring[slot] = k_frag(HALF, slot);
 #pragma unroll
         for (int u = 0; u < 16 / KS; u++) {
@@ -521,15 +539,12 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   };
 
   FA2_STAMP(1);
-  for (int t = 0; t < n_tiles; t++) {
-    step(2 * t, std::integral_constant<int, 0>{});
-    step(2 * t + 1, std::integral_constant<int, 1>{});
-    // Every wave is done with K_t and V_t; K_{t+2} and V_{t+1} (issued one tile ago) have landed.
+  // End of a tile: every wave is done with V_t and the K fragments of tile t+1 are in flight or
+  // in registers; K_{t+2} and V_{t+1} (issued during this tile) have landed.  Then the fragment
+  // pointers advance to K tile t+2 and V tile t+1 (stages are used round-robin).
+  auto end_tile = [&](int t) {
     wait_vmem_all();
     __syncthreads();
-    if (t + 3 < n_tiles) issue_k(t + 3);
-    if (t + 2 < n_tiles) issue_v(t + 2);
-    // Advance the fragment pointers to K tile t+2 and V tile t+1 (stages are used round-robin).
     const int dk = ((t + 2) % L::K_STAGES == 0) ? -(L::K_STAGES - 1) * L::TILE_ELEMS : L::TILE_ELEMS;
     const int dv = ((t + 1) % L::V_STAGES == 0) ? -(L::V_STAGES - 1) * L::TILE_ELEMS : L::TILE_ELEMS;
 #pragma unroll
@@ -539,6 +554,22 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
       vlo[db] += dv;
       vhi[db] += dv;
     }
+  };
+  int t = 0;
+  // Tiles whose loads are whole tiles inside the keys: spread over the first step.
+  const int n_spread = min(n_tiles, n_inside) - 2;
+  for (; t < n_spread; t++) {
+    step(2 * t, std::integral_constant<int, 0>{}, std::true_type{});
+    step(2 * t + 1, std::integral_constant<int, 1>{}, std::false_type{});
+    end_tile(t);
+  }
+  // The last tiles: whatever is left to load (possibly a ragged tile) is issued at once.
+  for (; t < n_tiles; t++) {
+    if (t + 2 < n_tiles) issue_k(t + 2);
+    if (t + 1 < n_tiles) issue_v(t + 1);
+    step(2 * t, std::integral_constant<int, 0>{}, std::false_type{});
+    step(2 * t + 1, std::integral_constant<int, 1>{}, std::false_type{});
+    end_tile(t);
   }
 
   FA2_STAMP(2);
