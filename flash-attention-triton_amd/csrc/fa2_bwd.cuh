@@ -691,6 +691,35 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
 // (Q rows -> dO rows -> dO^T -> Q^T -> next block's Q rows), the exponentials are issued under the
 // dP MFMAs and the dS arithmetic under the dV MFMAs.  Blocks on the diagonal (and a ragged last
 // tile) take the same code with the masks switched on.
+// MFMA whose accumulator is held in vector registers.  At one wave per SIMD the compiler gives every
+// MFMA result an accumulation register and copies it out (v_accvgpr_read) before vector
+// instructions can use it; S and dP are consumed by vector instructions right away, so their
+// chains are written out by hand with vector-register accumulators (dK and dV, which are only
+// read at the very end, stay in accumulation registers).  The compiler does not know these are
+// MFMAs: `settle` supplies the wait states an 8-pass MFMA result needs before vector
+// instructions may read it (11; the s_nop gives 12) and ties them to the value.
+template <typename T>
+struct VgprMfma;
+template <>
+struct VgprMfma<__bf16> {
+  static __device__ __forceinline__ void first(f32x16 &d, s16x8 a, s16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void next(f32x16 &d, s16x8 a, s16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+  }
+};
+template <>
+struct VgprMfma<_Float16> {
+  static __device__ __forceinline__ void first(f32x16 &d, s16x8 a, s16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void next(f32x16 &d, s16x8 a, s16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+  }
+};
+__device__ __forceinline__ void settle(f32x16 &d) { asm volatile("s_nop 11" : "+v"(d)); }
+
 template <int DP, int BQ>
 struct DkvDirectLayout {
   static constexpr int TILE_ELEMS = BQ * DP;
@@ -838,7 +867,6 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       dkacc[db][i] = 0.f;
       dvacc[db][i] = 0.f;
     }
-  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const int kvcol = kv0w + c;
 
 #pragma unroll
@@ -880,11 +908,12 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     typedef const __attribute__((address_space(3))) f32x4 *stat4_ptr;
 
     // ---- S = Q K^T (ring: Q rows -> dO rows); statistics of the 16 rows this lane holds -----
-    f32x16 s = zero, dp = zero;
+    f32x16 s, dp;
     f32x4 l4[4], d4[4];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      s = Elem<T>::mfma(ring[ks], kf[ks], s);
+      if (ks == 0) VgprMfma<T>::first(s, ring[ks], kf[ks]);
+      else VgprMfma<T>::next(s, ring[ks], kf[ks]);
       spread_load(ks);
       ring[ks] = lds_read_128(qrow[ks] + GOFF);
       constexpr int PER = (4 + KS - 1) / KS;  // row groups of four fetched per unit
@@ -902,13 +931,15 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     f32x16 pr;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      dp = Elem<T>::mfma(ring[ks], vf[ks], dp);
+      if (ks == 0) VgprMfma<T>::first(dp, ring[ks], vf[ks]);
+      else VgprMfma<T>::next(dp, ring[ks], vf[ks]);
       spread_load(KS + ks);
       {
         s16x4 a0 = lds_read_tr(qlo[ks % DB] + GOFF + 16 * (ks / DB) * DP);
         s16x4 a1 = lds_read_tr(qhi[ks % DB] + GOFF + 16 * (ks / DB) * DP);
         ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
+      if (ks == 0) settle(s);  // after the S chain's last MFMA and before the first read of S
 #pragma unroll
       for (int u = 0; u < 16 / KS; u++) {
         const int i = (16 / KS) * ks + u;
@@ -936,6 +967,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
         s16x4 a1 = lds_read_tr(qhi[ks % DB] + QOFF + 16 * (ks / DB) * DP);
         ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
+      if (ks == 0) settle(dp);
 #pragma unroll
       for (int u = 0; u < 16 / KS; u++) {
         const int i = (16 / KS) * ks + u;
