@@ -687,9 +687,11 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
 // The wave runs at one wave per SIMD (dK^T and dV^T alone are 128 accumulator registers), so
 // latency is hidden inside the wave: per 32-row query block the four GEMMs run back to back,
 //     S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS,
-// their A fragments travel through a ring of DP/16 register sets refilled as it is consumed
-// (Q rows -> dO rows -> dO^T -> Q^T -> next block's Q rows), the exponentials are issued under the
-// dP MFMAs and the dS arithmetic under the dV MFMAs.  Blocks on the diagonal (and a ragged last
+// their A fragments travel through two rings of DP/16 register sets, each refilled as it is
+// consumed with what the GEMM after next needs (ring: Q rows -> dO^T -> next block's Q rows;
+// ringb: dO rows -> Q^T -> next block's dO rows), so that every fragment is requested two GEMMs
+// before its MFMA; the exponentials are issued under the dP MFMAs and the dS arithmetic under the
+// dV MFMAs.  Blocks on the diagonal (and a ragged last
 // tile) take the same code with the masks switched on.
 // MFMA whose accumulator is held in vector registers.  At one wave per SIMD the compiler gives every
 // MFMA result an accumulation register and copies it out (v_accvgpr_read) before vector
@@ -879,10 +881,12 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   __syncthreads();
 
   FA2_STAMP(1);
-  // Ring of A fragments, preloaded with the Q rows of block 0.
-  s16x8 ring[KS];
+  // Two rings of A fragments, preloaded with the Q rows and the dO rows of block 0.
+  s16x8 ring[KS], ringb[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) ring[ks] = lds_read_128(qrow[ks]);
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) ringb[ks] = lds_read_128(qrow[ks] + L::TILE_ELEMS);
 
   // One 32-row query block.  HALF selects the half-tile; MASKED switches the causal/row masks on.
   // With SPREAD the block also issues the global->LDS loads of tile `lt`, one every fourth unit:
@@ -907,7 +911,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     constexpr int GOFF = QOFF + L::TILE_ELEMS;    // dO rows of this block
     typedef const __attribute__((address_space(3))) f32x4 *stat4_ptr;
 
-    // ---- S = Q K^T (ring: Q rows -> dO rows); statistics of the 16 rows this lane holds -----
+    // ---- S = Q K^T (ring: Q rows -> dO^T); statistics of the 16 rows this lane holds ---------
     f32x16 s, dp;
     f32x4 l4[4], d4[4];
 #pragma unroll
@@ -915,7 +919,11 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       if (ks == 0) VgprMfma<T>::first(s, ring[ks], kf[ks]);
       else VgprMfma<T>::next(s, ring[ks], kf[ks]);
       spread_load(ks);
-      ring[ks] = lds_read_128(qrow[ks] + GOFF);
+      {
+        s16x4 a0 = lds_read_tr(qlo[ks % DB] + GOFF + 16 * (ks / DB) * DP);
+        s16x4 a1 = lds_read_tr(qhi[ks % DB] + GOFF + 16 * (ks / DB) * DP);
+        ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
       constexpr int PER = (4 + KS - 1) / KS;  // row groups of four fetched per unit
 #pragma unroll
       for (int u = 0; u < PER; u++) {
@@ -927,17 +935,17 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    // ---- dP = dO V^T (ring: dO rows -> dO^T); exponentials under the MFMAs -------------------
+    // ---- dP = dO V^T (ringb: dO rows -> Q^T); exponentials under the MFMAs -------------------
     f32x16 pr;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      if (ks == 0) VgprMfma<T>::first(dp, ring[ks], vf[ks]);
-      else VgprMfma<T>::next(dp, ring[ks], vf[ks]);
+      if (ks == 0) VgprMfma<T>::first(dp, ringb[ks], vf[ks]);
+      else VgprMfma<T>::next(dp, ringb[ks], vf[ks]);
       spread_load(KS + ks);
       {
-        s16x4 a0 = lds_read_tr(qlo[ks % DB] + GOFF + 16 * (ks / DB) * DP);
-        s16x4 a1 = lds_read_tr(qhi[ks % DB] + GOFF + 16 * (ks / DB) * DP);
-        ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+        s16x4 a0 = lds_read_tr(qlo[ks % DB] + QOFF + 16 * (ks / DB) * DP);
+        s16x4 a1 = lds_read_tr(qhi[ks % DB] + QOFF + 16 * (ks / DB) * DP);
+        ringb[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
       if (ks == 0) settle(s);  // after the S chain's last MFMA and before the first read of S
 #pragma unroll
@@ -956,17 +964,13 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     f32x8 plo = {pr[0], pr[1], pr[2], pr[3], pr[4], pr[5], pr[6], pr[7]};
     f32x8 phi = {pr[8], pr[9], pr[10], pr[11], pr[12], pr[13], pr[14], pr[15]};
     const s16x8 pf[2] = {Elem<T>::pack8(plo), Elem<T>::pack8(phi)};
-    // ---- dV^T += dO^T P (ring: dO^T -> Q^T); dS arithmetic under the MFMAs --------------------
+    // ---- dV^T += dO^T P (ring: dO^T -> Q rows of the next block); dS arithmetic under the MFMAs
     f32x16 ds;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       dvacc[ks % DB] = Elem<T>::mfma(ring[ks], pf[ks / DB], dvacc[ks % DB]);
       spread_load(2 * KS + ks);
-      {
-        s16x4 a0 = lds_read_tr(qlo[ks % DB] + QOFF + 16 * (ks / DB) * DP);
-        s16x4 a1 = lds_read_tr(qhi[ks % DB] + QOFF + 16 * (ks / DB) * DP);
-        ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
-      }
+      ring[ks] = lds_read_128(qnext[ks] + (HALF == 0 ? 32 * DP : 0));
       if (ks == 0) settle(dp);
 #pragma unroll
       for (int u = 0; u < 16 / KS; u++) {
@@ -979,12 +983,12 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     f32x8 dlo = {ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]};
     f32x8 dhi = {ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]};
     const s16x8 dsf[2] = {Elem<T>::pack8(dlo), Elem<T>::pack8(dhi)};
-    // ---- dK^T += Q^T dS (ring: Q^T -> Q rows of the next block) --------------------------------
+    // ---- dK^T += Q^T dS (ringb: Q^T -> dO rows of the next block) ------------------------------
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      dkacc[ks % DB] = Elem<T>::mfma(ring[ks], dsf[ks / DB], dkacc[ks % DB]);
+      dkacc[ks % DB] = Elem<T>::mfma(ringb[ks], dsf[ks / DB], dkacc[ks % DB]);
       spread_load(3 * KS + ks);
-      ring[ks] = lds_read_128(qnext[ks] + (HALF == 0 ? 32 * DP : 0));
+      ringb[ks] = lds_read_128(qnext[ks] + L::TILE_ELEMS + (HALF == 0 ? 32 * DP : 0));
       __builtin_amdgcn_sched_barrier(0);
     }
   };
