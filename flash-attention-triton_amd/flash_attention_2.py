@@ -38,7 +38,13 @@ def _strides3(t: torch.Tensor) -> tuple[int, int, int]:
     return t.stride(0), t.stride(1), t.stride(2)
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_handle() -> int:
+    """hipStream_t of torch's current stream on the current device, as an integer."""
+    if _RAW_STREAM is not None:  # same value as below without building a Stream object (~10 us)
+        return _RAW_STREAM(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -324,6 +330,24 @@ def _validate_runtime_compatibility(cc: tuple[int, int], arch_name: str | None =
     _capi.load()  # raises RuntimeError when the library is missing or has the wrong ABI
 
 
+_VALIDATED_DEVICES: dict[int, tuple[int, int]] = {}
+
+
+def _validated_capability() -> tuple[int, int]:
+    """Compute capability of the current device, checked once per device.
+
+    The two device queries behind the check cost about 20 us per call, which is as much as the
+    rest of the forward wrapper; a device that passed keeps passing, one that failed is asked again.
+    """
+    index = torch.cuda.current_device()
+    cc = _VALIDATED_DEVICES.get(index)
+    if cc is None:
+        cc = torch.cuda.get_device_capability(index)
+        _validate_runtime_compatibility(cc)
+        _VALIDATED_DEVICES[index] = cc
+    return cc
+
+
 def _select_optimal_gpu_architecture(cc: tuple[int, int], deterministic: bool) -> KernelsConfigV2:
     """Pick the configuration for the device (reference: flash_attention_2.py:617-642).
 
@@ -357,8 +381,7 @@ def flash_attention_v2(
     Returns:
         Attention output tensor, same shape and dtype as q.
     """
-    cc = torch.cuda.get_device_capability()
-    _validate_runtime_compatibility(cc)
+    cc = _validated_capability()
 
     kernels_config = _select_optimal_gpu_architecture(cc, deterministic)
 
