@@ -283,6 +283,14 @@ template <typename T, int DP, int BQ>
 __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdParams p) {
   using L = DkvLayout<DP, BQ>;
   constexpr int KS = DP / 16, DB = DP / 32, MQ = BQ / 32, CPR = DP / 8;
+  // At 256 columns the two accumulators (2 x 128 registers) no longer fit beside the K and V
+  // fragments (another 128): the head dimension is then covered in two passes over the query tiles,
+  // each accumulating half of the columns of dK and dV (S and dP are formed again in the second
+  // pass).  Measured at B=2, H=8, N=4096: 811 us against 2273 us with one pass and 1 KiB of
+  // spills per lane; at 192 columns one pass is the faster (295 us against 640 us).
+  constexpr int NPASS = DP > 192 ? 2 : 1;
+  constexpr int DBP = DB / NPASS;  // 32-column blocks of dK / dV per pass
+  static_assert(DB % NPASS == 0, "passes must split the head dimension evenly");
   constexpr int NTHREADS = 64 * kDkvWaves;
   constexpr int CPT = (BQ * CPR) / NTHREADS;
   static_assert((BQ * CPR) % NTHREADS == 0, "tile must split evenly over the workgroup");
@@ -367,9 +375,15 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdPa
     }
   };
 
-  f32x16 dkacc[DB], dvacc[DB];
+  const int row_frag_off = c * L::QLD + 8 * h;
+  const int tr_frag_off = (4 * h + (i16 >> 2)) * L::QLD + 16 * g2 + 4 * (i16 & 3);
+  const int kvcol = kv0w + c;
+
+  for (int pass = 0; pass < NPASS; pass++) {
+  const int col0 = pass * DBP * 32;  // first dK / dV column of this pass
+  f32x16 dkacc[DBP], dvacc[DBP];
 #pragma unroll
-  for (int db = 0; db < DB; db++)
+  for (int db = 0; db < DBP; db++)
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       dkacc[db][i] = 0.f;
@@ -382,15 +396,14 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdPa
   }
   __syncthreads();
 
-  const int row_frag_off = c * L::QLD + 8 * h;
-  const int tr_frag_off = (4 * h + (i16 >> 2)) * L::QLD + 16 * g2 + 4 * (i16 & 3);
-  const int kvcol = kv0w + c;
-
   for (int t = 0; t < n_tiles; t++) {
     const int buf = t & 1;
     const int qt0 = q_begin + t * BQ;
     const bool more = (t + 1) < n_tiles;
-    if (more) load_tile(qt0 + BQ);
+    // The next tile travels through registers while this one is worked on, except at 256
+    // columns, where those registers are not to be had: there it is fetched after the MFMAs.
+    constexpr bool EARLY_LOAD = DP <= 192;
+    if (EARLY_LOAD && more) load_tile(qt0 + BQ);
 
     const short *sq = smem + buf * L::STAGE_ELEMS;
     const short *sg = sq + L::Q_ELEMS;
@@ -444,8 +457,8 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdPa
 #pragma unroll
         for (int tt = 0; tt < 2; tt++) {
 #pragma unroll
-          for (int db = 0; db < DB; db++) {
-            const int off = tr_frag_off + (32 * mq + 16 * tt) * L::QLD + 32 * db;
+          for (int db = 0; db < DBP; db++) {
+            const int off = tr_frag_off + (32 * mq + 16 * tt) * L::QLD + col0 + 32 * db;
             s16x8 ag = lds_read_tr_frag(sg + off, L::QLD);
             dvacc[db] = Elem<T>::mfma(ag, pf[tt], dvacc[db]);
             s16x8 aq = lds_read_tr_frag(sq + off, L::QLD);
@@ -455,19 +468,27 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdPa
       }
     }
 
+    if (!EARLY_LOAD && more) load_tile(qt0 + BQ);
     if (more) store_tile(buf ^ 1);
     __syncthreads();
   }
 
+  // Columns [col0, col0 + 32 DBP) of this wave's 32 rows of dV and dK.  The patch overlays the
+  // stages: the loop's last barrier ordered it after all reads, and the barrier below orders the
+  // next pass's tile stores after it.
   short *patch = smem + wave * 32 * (DP + 8);
-  store_transposed_acc<T, DP>(dvacc, 1.0f, patch, DV + (int64_t)kv0w * p.dv.stride_seq,
-                              p.dv.stride_seq, p.seqlen_k - kv0w, p.headdim, vec);
+  store_transposed_acc<T, 32 * DBP>(dvacc, 1.0f, patch, DV + (int64_t)kv0w * p.dv.stride_seq + col0,
+                                    p.dv.stride_seq, p.seqlen_k - kv0w, p.headdim - col0, vec);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  store_transposed_acc<T, DP>(dkacc, p.scale, patch, DK + (int64_t)kv0w * p.dk.stride_seq,
-                              p.dk.stride_seq, p.seqlen_k - kv0w, p.headdim, vec);
+  store_transposed_acc<T, 32 * DBP>(dkacc, p.scale, patch, DK + (int64_t)kv0w * p.dk.stride_seq + col0,
+                                    p.dk.stride_seq, p.seqlen_k - kv0w, p.headdim - col0, vec);
+  if (pass + 1 < NPASS) __syncthreads();
+  }
 }
+
+
 
 // ------------------------------------------------------------------------------------------
 // Fast paths (head dimension equal to the padded one, 16-byte aligned rows): the streamed tiles
