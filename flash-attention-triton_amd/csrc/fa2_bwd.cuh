@@ -497,13 +497,17 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdPa
 // ------------------------------------------------------------------------------------------
 __device__ __forceinline__ void bwd_wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+// K tiles in three stages and V tiles in two, like the forward: tile t brings in K tile t+2 and V
+// tile t+1, so that the K rows of the next tile are there when the last block of a tile fetches them.
 template <int DP, int BKV>
 struct DqDirectLayout {
   static constexpr int TILE_ELEMS = BKV * DP;
-  static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;  // K tile then V tile
+  static constexpr int K_STAGES = 3, V_STAGES = 2;
+  static constexpr int K_BASE = 0;
+  static constexpr int V_BASE = K_STAGES * TILE_ELEMS;
+  static constexpr int STAGE_ELEMS = (K_STAGES + V_STAGES) * TILE_ELEMS;
   static constexpr int PATCH_ELEMS = kDqWaves * 32 * (DP + 8);
-  static constexpr int TOTAL_ELEMS =
-      (2 * STAGE_ELEMS > PATCH_ELEMS) ? 2 * STAGE_ELEMS : PATCH_ELEMS;
+  static constexpr int TOTAL_ELEMS = (STAGE_ELEMS > PATCH_ELEMS) ? STAGE_ELEMS : PATCH_ELEMS;
 };
 
 // With FUSE_DELTA the kernel also computes delta = rowsum(O * dO) for its query rows (it holds
@@ -549,18 +553,18 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   const int n_inside = seqlen_k / BKV;
 
   const unsigned lds_base = lds_u32(smem);  // LDS byte address of smem
-  auto issue_tile = [&](int t) {
-    const unsigned dst = lds_base + 2u * (unsigned)((t & 1) * L::STAGE_ELEMS);
-    if (t < n_inside) {
-      kload.issue(t * BKV, dst);
-      vload.issue(t * BKV, dst + 2u * L::TILE_ELEMS);
-    } else {
-      kload.issue_clamped(t * BKV, seqlen_k, dst);
-      vload.issue_clamped(t * BKV, seqlen_k, dst + 2u * L::TILE_ELEMS);
-    }
+  auto issue_k = [&](int t) {
+    const unsigned dst = lds_base + 2u * (unsigned)(L::K_BASE + (t % L::K_STAGES) * L::TILE_ELEMS);
+    if (t < n_inside) kload.issue(t * BKV, dst); else kload.issue_clamped(t * BKV, seqlen_k, dst);
   };
-  issue_tile(0);
-  if (n_tiles > 1) issue_tile(1);
+  auto issue_v = [&](int t) {
+    const unsigned dst = lds_base + 2u * (unsigned)(L::V_BASE + (t % L::V_STAGES) * L::TILE_ELEMS);
+    if (t < n_inside) vload.issue(t * BKV, dst); else vload.issue_clamped(t * BKV, seqlen_k, dst);
+  };
+  // K_0, V_0 and K_1 are loaded here; after that tile t brings in K_{t+2} and V_{t+1}.
+  issue_k(0);
+  issue_v(0);
+  if (n_tiles > 1) issue_k(1);
 
   // B operands: lane (c, h) holds row q0w + c of Q and of dO, columns 16 ks + 8 h + j.
   s16x8 qf[KS], gf[KS];
@@ -596,19 +600,23 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
     }
   }
 
-  // Swizzled fragment addresses inside stage 0 (32-bit LDS pointers).
+  // Swizzled fragment addresses (32-bit LDS pointers).  knext: K rows of the tile the next block
+  // lies in; vrow: V rows of the current tile; klo/khi: transposed K fragments of the current tile.
   const lds_cptr lds0 = to_lds(smem);
-  lds_cptr krow[KS], klo[DB], khi[DB];
+  lds_cptr knext[KS], vrow[KS], klo[DB], khi[DB];
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) krow[ks] = lds0 + swz_off<DP>(c, 2 * ks + h);
+  for (int ks = 0; ks < KS; ks++) {
+    knext[ks] = lds0 + L::K_BASE + swz_off<DP>(c, 2 * ks + h);
+    vrow[ks] = lds0 + L::V_BASE + swz_off<DP>(c, 2 * ks + h);
+  }
   {
     const int rowlo = 4 * h + (i16 >> 2);
     const int sub = (i16 & 1) * 4;
 #pragma unroll
     for (int db = 0; db < DB; db++) {
       const int chunk = 4 * db + 2 * g2 + ((i16 & 3) >> 1);
-      klo[db] = lds0 + swz_off<DP>(rowlo, chunk) + sub;
-      khi[db] = lds0 + swz_off<DP>(rowlo + 8, chunk) + sub;
+      klo[db] = lds0 + L::K_BASE + swz_off<DP>(rowlo, chunk) + sub;
+      khi[db] = lds0 + L::K_BASE + swz_off<DP>(rowlo + 8, chunk) + sub;
     }
   }
 
@@ -623,97 +631,127 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   bwd_wait_vmem_all();
   __syncthreads();
 
-  // Tiles [1, n_spread) bring in their successor during their first block, one global->LDS load
-  // every other MFMA of the first two GEMMs: issued back to back by all waves after a barrier the
-  // loads queue up in the memory pipeline, and a wave whose load cannot issue cannot issue its
-  // MFMAs either.  The other tiles' successors (ragged tiles, and tile 1) are loaded at once.
+  // Ring of A fragments, preloaded with the K rows of block 0.
+  s16x8 ring[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) ring[ks] = lds_read_128(knext[ks]);
+
+  // One 32-key block j = 2 t + HALF, three GEMMs of KS MFMAs, each unit = one MFMA, the LDS reads
+  // that refill the ring slot it freed, and a share of the vector work:
+  //     A: S^T = K Q^T            ring <- V rows              (loads of V tile t+1 when SPREAD)
+  //     B: dP^T = V dO^T          ring <- K^T fragments       exponentials of S; loads of K tile t+2
+  //     C: dQ^T += K^T dS^T       ring <- next block's K rows second half of the dS arithmetic
   constexpr int LOADS = TileLoader<DP, BKV, kDqWaves>::LOADS;
-  static_assert(KS >= 2 * LOADS, "the first two GEMMs have a slot for every load");
-  const int n_spread = min(n_tiles, n_inside) - 1;
-  auto tile = [&](int t, auto spread_tag) {
+  constexpr int LOAD_EVERY = KS / LOADS;
+  auto block = [&](int j, auto half_tag, auto spread_tag) __attribute__((always_inline)) {
+    constexpr int HALF = decltype(half_tag)::value;
     constexpr bool SPREAD = decltype(spread_tag)::value;
-    const int soff = (t & 1) * L::STAGE_ELEMS;
-    const unsigned ldst = lds_base + 2u * (unsigned)(((t + 1) & 1) * L::STAGE_ELEMS);
-    // Load li of the 2 LOADS that make up K tile t+1 and V tile t+1.
-    auto spread_load = [&](int li) {
-      if (li < LOADS) kload.issue_one((t + 1) * BKV, ldst, li);
-      else if (li < 2 * LOADS) vload.issue_one((t + 1) * BKV, ldst + 2u * L::TILE_ELEMS, li - LOADS);
-    };
-#pragma unroll
-    for (int mb = 0; mb < 2; mb++) {
-      const int j = 2 * t + mb;
-      const bool spread_here = SPREAD && mb == 0;
-      if (j < n_mine) {
-        const int koff = soff + mb * BLK * DP;
-        const int voff = koff + L::TILE_ELEMS;
-        f32x16 s = zero, dp = zero;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-          s = Elem<T>::mfma(lds_read_128(krow[ks] + koff), qf[ks], s);
-          if (spread_here && ks % 2 == 0) spread_load(ks / 2);
-        }
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-          dp = Elem<T>::mfma(lds_read_128(krow[ks] + voff), gf[ks], dp);
-          if (spread_here && ks % 2 == 0) spread_load(KS / 2 + ks / 2);
-        }
-        const bool need_mask = j >= n_full;
-        f32x16 ds;
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          float pr = fast_exp2(s[i] * scale_log2 - lse2);
-          if (need_mask) {
-            const int kv = j * BLK + 8 * (i >> 2) + 4 * h + (i & 3);
-            if (kv > qrow || kv >= seqlen_k) pr = 0.f;
-          }
-          ds[i] = pr * (dp[i] - delta);
-        }
-        f32x8 lo = {ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]};
-        f32x8 hi = {ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]};
-        const s16x8 dsf[2] = {Elem<T>::pack8(lo), Elem<T>::pack8(hi)};
-#pragma unroll
-        for (int ks2 = 0; ks2 < 2; ks2++) {
-#pragma unroll
-          for (int db = 0; db < DB; db++) {
-            s16x4 a0 = lds_read_tr(klo[db] + koff + 16 * ks2 * DP);
-            s16x4 a1 = lds_read_tr(khi[db] + koff + 16 * ks2 * DP);
-            s16x8 a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
-            dqacc[db] = Elem<T>::mfma(a, dsf[ks2], dqacc[db]);
-          }
-        }
-      } else if (spread_here) {  // not reached: skipped blocks lie in the last two tiles
-        issue_tile(t + 1);
+    const int kt = j / 2 + 2, vt = j / 2 + 1;  // tiles loaded during this block (SPREAD)
+    if (j >= n_mine) {
+      if (SPREAD) {  // not reached: skipped blocks lie in the last two tiles, which load nothing
+        issue_k(kt);
+        issue_v(vt);
       }
+      return;
     }
-    // Everyone is done with stage t & 1; tile t+1 (issued during this tile or before) has landed.
+    const unsigned kdst = lds_base + 2u * (unsigned)(L::K_BASE + (kt % L::K_STAGES) * L::TILE_ELEMS);
+    const unsigned vdst = lds_base + 2u * (unsigned)(L::V_BASE + (vt % L::V_STAGES) * L::TILE_ELEMS);
+    constexpr int HOFF = HALF * BLK * DP;
+    f32x16 s = zero, dp = zero;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      s = Elem<T>::mfma(ring[ks], qf[ks], s);
+      if (SPREAD && ks % LOAD_EVERY == 0) vload.issue_one(vt * BKV, vdst, ks / LOAD_EVERY);
+      ring[ks] = lds_read_128(vrow[ks] + HOFF);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const bool need_mask = j >= n_full;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      dp = Elem<T>::mfma(ring[ks], gf[ks], dp);
+      if (SPREAD && ks % LOAD_EVERY == 0) kload.issue_one(kt * BKV, kdst, ks / LOAD_EVERY);
+      {
+        s16x4 a0 = lds_read_tr(klo[ks % DB] + HOFF + 16 * (ks / DB) * DP);
+        s16x4 a1 = lds_read_tr(khi[ks % DB] + HOFF + 16 * (ks / DB) * DP);
+        ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+#pragma unroll
+      for (int u = 0; u < 16 / KS; u++) {
+        const int i = (16 / KS) * ks + u;
+        float pr = fast_exp2(s[i] * scale_log2 - lse2);
+        if (need_mask) {
+          const int kv = j * BLK + 8 * (i >> 2) + 4 * h + (i & 3);
+          if (kv > qrow || kv >= seqlen_k) pr = 0.f;
+        }
+        s[i] = pr;
+      }
+      asm volatile("" : "+v"(s));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // dS of the first 16 keys before the dQ MFMAs that need them, the rest beside those MFMAs.
+    f32x8 lo, hi;
+#pragma unroll
+    for (int i = 0; i < 8; i++) lo[i] = s[i] * (dp[i] - delta);
+    s16x8 dsf[2];
+    dsf[0] = Elem<T>::pack8(lo);
+#pragma unroll
+    for (int slot = 0; slot < KS; slot++) {
+      constexpr int HALF_SLOTS = KS / 2;
+      const int ks2 = slot / DB, db = slot % DB;
+      dqacc[db] = Elem<T>::mfma(ring[slot], dsf[ks2], dqacc[db]);
+      ring[slot] = lds_read_128(knext[slot] + (HALF == 0 ? BLK * DP : 0));
+      if (slot < HALF_SLOTS) {
+#pragma unroll
+        for (int u = 0; u < 8 / HALF_SLOTS; u++) {
+          const int i = (8 / HALF_SLOTS) * slot + u;
+          hi[i] = s[8 + i] * (dp[8 + i] - delta);
+        }
+        asm volatile("" : "+v"(hi));
+        if (slot == HALF_SLOTS - 1) dsf[1] = Elem<T>::pack8(hi);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // End of a tile: every wave is done with V_t and with K_t; K_{t+2} and V_{t+1} (issued during
+  // this tile) have landed.  The fragment pointers advance (stages are used round-robin).
+  auto k_step = [&](int t) { return ((t + 1) % L::K_STAGES == 0) ? -(L::K_STAGES - 1) * L::TILE_ELEMS : L::TILE_ELEMS; };
+  auto end_tile = [&](int t) {
     bwd_wait_vmem_all();
     __syncthreads();
-    if (t + 2 < n_tiles && t + 1 >= n_spread) issue_tile(t + 2);
+    const int dk = k_step(t);
+    const int dv = ((t + 1) % L::V_STAGES == 0) ? -(L::V_STAGES - 1) * L::TILE_ELEMS : L::TILE_ELEMS;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) vrow[ks] += dv;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      klo[db] += dk;
+      khi[db] += dk;
+    }
+  };
+  auto tile = [&](int t, auto spread_tag) __attribute__((always_inline)) {
+    block(2 * t, std::integral_constant<int, 0>{}, spread_tag);
+    // knext -> K tile t+1 before the second block prefetches from it.
+    const int dk = k_step(t);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) knext[ks] += dk;
+    block(2 * t + 1, std::integral_constant<int, 1>{}, std::false_type{});
+    end_tile(t);
   };
   int t = 0;
-  if (n_tiles > 0) {  // tile 1 was loaded before the loop
-    tile(0, std::false_type{});
-    t = 1;
-  }
+  const int n_spread = min(n_tiles, n_inside) - 2;
   for (; t < n_spread; t++) tile(t, std::true_type{});
-  for (; t < n_tiles; t++) tile(t, std::false_type{});
+  for (; t < n_tiles; t++) {
+    if (t + 2 < n_tiles) issue_k(t + 2);
+    if (t + 1 < n_tiles) issue_v(t + 1);
+    tile(t, std::false_type{});
+  }
 
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(dqacc, p.scale, patch, DQ + (int64_t)q0w * p.dq.stride_seq,
                               p.dq.stride_seq, p.seqlen_q - q0w, DP, true);
 }
 
-// dK/dV fast path.  One workgroup per 128 key rows, one wave per 32 of them (K and V fragments in
-// registers); Q and dO tiles of 64 rows stream through three LDS stages (one barrier per tile).
-// The wave runs at one wave per SIMD (dK^T and dV^T alone are 128 accumulator registers), so
-// latency is hidden inside the wave: per 32-row query block the four GEMMs run back to back,
-//     S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS,
-// their A fragments travel through two rings of DP/16 register sets, each refilled as it is
-// consumed with what the GEMM after next needs (ring: Q rows -> dO^T -> next block's Q rows;
-// ringb: dO rows -> Q^T -> next block's dO rows), so that every fragment is requested two GEMMs
-// before its MFMA; the exponentials are issued under the dP MFMAs and the dS arithmetic under the
-// dV MFMAs.  Blocks on the diagonal (and a ragged last
-// tile) take the same code with the masks switched on.
 // MFMA whose accumulator is held in vector registers.  At one wave per SIMD the compiler gives every
 // MFMA result an accumulation register and copies it out (v_accvgpr_read) before vector
 // instructions can use it; S and dP are consumed by vector instructions right away, so their
