@@ -35,9 +35,9 @@ CALIBRATION_BYTES = 256 << 20
 # the summary sits in profiles/fwd_bwd_kernels_c3_bf16_hbm_traffic.txt.  Counters cannot be read
 # from inside the process, so other workloads report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("C3", "fwd"): 783.8e6,
-    ("C3", "bwd_dkdv"): 879.5e6,
-    ("C3", "bwd_dq"): 803.3e6,
+    ("C3", "fwd"): 776.7e6,
+    ("C3", "bwd_dkdv"): 878.5e6,
+    ("C3", "bwd_dq"): 842.2e6,
     ("C3", "bwd_preprocess"): 135.3e6,
 }
 PEAK_HBM_GBS = 8000.0
