@@ -11,7 +11,7 @@ LIBRARY = CSRC / "libfa2_gfx950.so"
 
 def build(force: bool = True) -> pathlib.Path:
     """Compile the HIP kernels and the C ABI.  ``force`` rebuilds even if the library exists."""
-    cmd = ["make", "-C", str(CSRC)]
+    cmd = ["make", "-j4", "-C", str(CSRC)]
     if force:
         cmd.append("-B")
     subprocess.run(cmd, check=True)

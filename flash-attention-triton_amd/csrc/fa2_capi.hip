@@ -10,8 +10,7 @@
 #include <cstdarg>
 #include <cstdio>
 
-#include "fa2_bwd.cuh"
-#include "fa2_fwd.cuh"
+#include "fa2_launch.hpp"
 
 namespace {
 
@@ -28,9 +27,9 @@ int fail(int status, const char *fmt, ...) {
 // ---- gfx950 tile/wave table -----------------------------------------------------------------
 // One row per padded head dimension.  All rows use 4 waves of 64 lanes per workgroup and the
 // 32x32x16 MFMA; a wave always owns 32 sequence positions of the operand it keeps in registers.
-constexpr int kFwdBlockKV = 64;
-constexpr int kDqBlockKV = 64;
-constexpr int kDkvBlockQ = 64;
+using fa2::kDkvBlockQ;
+using fa2::kDqBlockKV;
+using fa2::kFwdBlockKV;
 
 const fa2_config_info kTable[] = {
     // id  DP   fwd: BQ   BKV waves   dK/dV: BQ  BKV  waves   dQ: BQ  BKV  waves
@@ -100,92 +99,6 @@ int launch_status(const char *what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(FA2_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
   return FA2_OK;
-}
-
-template <typename T, bool VEC>
-void launch_fwd_v(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
-  dim3 block(64 * fa2::kFwdWaves);
-  switch (dp) {
-    case 32: hipLaunchKernelGGL((fa2::fwd_kernel<T, 32, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
-    case 64: hipLaunchKernelGGL((fa2::fwd_kernel<T, 64, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
-    case 96: hipLaunchKernelGGL((fa2::fwd_kernel<T, 96, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
-    case 128: hipLaunchKernelGGL((fa2::fwd_kernel<T, 128, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
-    case 192: hipLaunchKernelGGL((fa2::fwd_kernel<T, 192, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fa2::fwd_kernel<T, 256, kFwdBlockKV, VEC>), grid, block, 0, s, p); break;
-  }
-}
-
-// The fast kernels need the exact padded head dimension, 16-byte aligned rows and row offsets
-// inside a tile that fit 32 bits.
-bool direct_ok(const fa2::Tensor4 &t) { return t.stride_seq < (int64_t(1) << 24); }
-
-template <typename T>
-void launch_fwd(int dp, const fa2::FwdParams &p, dim3 grid, hipStream_t s) {
-  dim3 block(64 * fa2::kFwdWaves);
-  if (p.vec && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128) && direct_ok(p.k) && direct_ok(p.v)) {
-    switch (dp) {
-      case 32: hipLaunchKernelGGL((fa2::fwd_direct_kernel<T, 32, kFwdBlockKV>), grid, block, 0, s, p); break;
-      case 64: hipLaunchKernelGGL((fa2::fwd_direct_kernel<T, 64, kFwdBlockKV>), grid, block, 0, s, p); break;
-      default: hipLaunchKernelGGL((fa2::fwd_direct_kernel<T, 128, kFwdBlockKV>), grid, block, 0, s, p); break;
-    }
-    return;
-  }
-  if (p.vec)
-    launch_fwd_v<T, true>(dp, p, grid, s);
-  else
-    launch_fwd_v<T, false>(dp, p, grid, s);
-}
-
-bool dq_direct_ok(int dp, const fa2::BwdParams &p) {
-  return p.vec && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128) && direct_ok(p.k) && direct_ok(p.v);
-}
-
-template <typename T, bool FUSE_DELTA>
-void launch_dq_direct(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
-  dim3 block(64 * fa2::kDqWaves);
-  switch (dp) {
-    case 32: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 32, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
-    case 64: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 64, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fa2::bwd_dq_direct_kernel<T, 128, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
-  }
-}
-
-template <typename T>
-void launch_dq(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
-  dim3 block(64 * fa2::kDqWaves);
-  if (dq_direct_ok(dp, p)) {
-    launch_dq_direct<T, false>(dp, p, grid, s);
-    return;
-  }
-  switch (dp) {
-    case 32: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 32, kDqBlockKV>), grid, block, 0, s, p); break;
-    case 64: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 64, kDqBlockKV>), grid, block, 0, s, p); break;
-    case 96: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 96, kDqBlockKV>), grid, block, 0, s, p); break;
-    case 128: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 128, kDqBlockKV>), grid, block, 0, s, p); break;
-    case 192: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 192, kDqBlockKV>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fa2::bwd_dq_kernel<T, 256, kDqBlockKV>), grid, block, 0, s, p); break;
-  }
-}
-
-template <typename T>
-void launch_dkdv(int dp, const fa2::BwdParams &p, dim3 grid, hipStream_t s) {
-  dim3 block(64 * fa2::kDkvWaves);
-  if (p.vec && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128) && direct_ok(p.q) && direct_ok(p.d_o)) {
-    switch (dp) {
-      case 32: hipLaunchKernelGGL((fa2::bwd_dkdv_direct_kernel<T, 32, kDkvBlockQ>), grid, block, 0, s, p); break;
-      case 64: hipLaunchKernelGGL((fa2::bwd_dkdv_direct_kernel<T, 64, kDkvBlockQ>), grid, block, 0, s, p); break;
-      default: hipLaunchKernelGGL((fa2::bwd_dkdv_direct_kernel<T, 128, kDkvBlockQ>), grid, block, 0, s, p); break;
-    }
-    return;
-  }
-  switch (dp) {
-    case 32: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 32, kDkvBlockQ>), grid, block, 0, s, p); break;
-    case 64: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 64, kDkvBlockQ>), grid, block, 0, s, p); break;
-    case 96: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 96, kDkvBlockQ>), grid, block, 0, s, p); break;
-    case 128: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 128, kDkvBlockQ>), grid, block, 0, s, p); break;
-    case 192: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 192, kDkvBlockQ>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fa2::bwd_dkdv_kernel<T, 256, kDkvBlockQ>), grid, block, 0, s, p); break;
-  }
 }
 
 }  // namespace
@@ -273,10 +186,7 @@ int fa2_fwd(const void *q, const void *k, const void *v, void *o, float *lse, in
   dim3 grid((unsigned)nwg);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const int dp = kTable[cfg].headdim_padded;
-  if (dtype == FA2_DTYPE_BF16)
-    launch_fwd<__bf16>(dp, p, grid, s);
-  else
-    launch_fwd<_Float16>(dp, p, grid, s);
+  fa2::launch_fwd(dtype == FA2_DTYPE_BF16, dp, p, grid, s);
   return launch_status("fa2_fwd launch");
 }
 
@@ -302,10 +212,7 @@ int fa2_bwd_preprocess(const void *o, const void *d_o, float *delta, int batch, 
   if (bh > 65535) return fail(FA2_ERR_TOO_LARGE, "batch*nheads=%lld exceeds the grid's second dimension", (long long)bh);
   dim3 grid((seqlen_q_rounded + 15) / 16, (unsigned)bh);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (dtype == FA2_DTYPE_BF16)
-    hipLaunchKernelGGL((fa2::bwd_preprocess_kernel<__bf16>), grid, dim3(256), 0, s, p);
-  else
-    hipLaunchKernelGGL((fa2::bwd_preprocess_kernel<_Float16>), grid, dim3(256), 0, s, p);
+  fa2::launch_preprocess(dtype == FA2_DTYPE_BF16, p, grid, s);
   return launch_status("fa2_bwd_preprocess launch");
 }
 
@@ -387,20 +294,14 @@ int bwd_impl(const void *q, const void *k, const void *v, const void *o, const v
 
   auto run_dkdv = [&]() {
     dim3 grid((unsigned)nwg_k);
-    if (dtype == FA2_DTYPE_BF16)
-      launch_dkdv<__bf16>(dp, pk, grid, s);
-    else
-      launch_dkdv<_Float16>(dp, pk, grid, s);
+    fa2::launch_dkdv(dtype == FA2_DTYPE_BF16, dp, pk, grid, s);
     return launch_status("fa2_bwd dK/dV launch");
   };
 
-  if (fused && dq_direct_ok(dp, pq) && vec_ok(p.o, headdim)) {
+  if (fused && fa2::dq_direct_ok(dp, pq) && vec_ok(p.o, headdim)) {
     // dQ first: it writes delta, which the dK/dV kernel reads.
     dim3 grid((unsigned)nwg_q);
-    if (dtype == FA2_DTYPE_BF16)
-      launch_dq_direct<__bf16, true>(dp, pq, grid, s);
-    else
-      launch_dq_direct<_Float16, true>(dp, pq, grid, s);
+    fa2::launch_dq(dtype == FA2_DTYPE_BF16, dp, pq, grid, true, s);
     if ((rc = launch_status("fa2_bwd_fused dQ launch"))) return rc;
     return run_dkdv();
   }
@@ -412,10 +313,7 @@ int bwd_impl(const void *q, const void *k, const void *v, const void *o, const v
   if (want_dkdv && (rc = run_dkdv())) return rc;
   if (want_dq) {
     dim3 grid((unsigned)nwg_q);
-    if (dtype == FA2_DTYPE_BF16)
-      launch_dq<__bf16>(dp, pq, grid, s);
-    else
-      launch_dq<_Float16>(dp, pq, grid, s);
+    fa2::launch_dq(dtype == FA2_DTYPE_BF16, dp, pq, grid, false, s);
     if ((rc = launch_status("fa2_bwd dQ launch"))) return rc;
   }
   return FA2_OK;
@@ -459,11 +357,5 @@ int fa2_bwd_fused(const void *q, const void *k, const void *v, const void *o, co
                   seqlen_q_rounded, st, o_st, softmax_scale, dtype, config_id, stream);
 }
 
-#ifdef FA2_WG_STAMPS
-// Debug build only (never declared in the public header): copies the workgroup stamps to the host.
-int fa2_debug_wg_stamps(long long *out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(fa2::fa2_wg_stamps), sizeof(long long) * 8192 * 4);
-}
-#endif
 
 }  // extern "C"

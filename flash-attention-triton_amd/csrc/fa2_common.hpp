@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fa2_params.hpp"
+
 namespace fa2 {
 
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -31,12 +33,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
-
-// One (batch, nheads, seqlen, headdim) tensor: base pointer and strides in elements.
-struct Tensor4 {
-  void *ptr;
-  int64_t stride_batch, stride_head, stride_seq;
-};
 
 template <typename T>
 struct Elem;
@@ -230,14 +226,6 @@ __device__ __forceinline__ void map_workgroup(int i, int heads, int tiles_per_he
   rank = r / gsize;
 }
 
-#ifdef FA2_WG_STAMPS
-// Debug build only: wall-clock (100 MHz) stamps per workgroup: start, loop start, loop end, end.
-__device__ long long fa2_wg_stamps[8192][4];
-#define FA2_STAMP(slot) do { if (threadIdx.x == 0 && blockIdx.x < 8192) fa2_wg_stamps[blockIdx.x][slot] = wall_clock64(); } while (0)
-#else
-#define FA2_STAMP(slot) do {} while (0)
-#endif
-
 }  // namespace fa2
 
 // ------------------------------------------------------------------------------------------
@@ -274,6 +262,9 @@ __device__ __forceinline__ int swz_off(int r, int c) { return r * DP + ((c ^ swz
 // LDS destinations are passed around as 32-bit byte addresses (wave-uniform integers): converting
 // a generic pointer into an LDS address costs a null check and 64-bit arithmetic per load, an
 // integer add does not.  lds_u32(p) does the conversion once.
+// M0 is overwritten without being named as a clobber: the gfx9 backend treats M0 as a reserved
+// register, sets it immediately before each of its own instructions that read it and never keeps
+// a value in it across other code (naming it only draws -Winline-asm "reserved register").
 __device__ __forceinline__ unsigned lds_u32(const short *p) {
   return (unsigned)__builtin_amdgcn_readfirstlane(
       (int)(unsigned)(uintptr_t)(__attribute__((address_space(3))) const void *)p);
@@ -305,6 +296,9 @@ __device__ __forceinline__ void load_lds_16(const short *uniform_base, unsigned 
       : "v"(lane_byte_offset), "s"(uniform_base), "s"(lds_wave_addr)
       : "memory");
 }
+
+// s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt fields left at their maxima).
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
 // Streams ROWS x DP tiles of a (seqlen, headdim) matrix into swizzled LDS with LDS-direct loads.
 // All NW waves of the workgroup take part; each wave issues LOADS loads of 1 KiB per tile.

@@ -24,22 +24,9 @@
 
 #include <type_traits>
 
-#include "fa2_common.cuh"
+#include "fa2_common.hpp"
 
 namespace fa2 {
-
-struct FwdParams {
-  Tensor4 q, k, v, o;
-  float *lse;
-  int batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded;
-  int n_qtiles;
-  float scale;       // softmax scale (natural units)
-  float scale_log2;  // scale * log2(e)
-  int vec;           // 16-byte global accesses are legal for every tensor
-};
-
-constexpr int kFwdWaves = 4;
-constexpr int kFwdBlockQ = 32 * kFwdWaves;
 
 // The running max is only raised (and the accumulator rescaled) when some row's new maximum
 // exceeds the one in use by more than this many powers of two; until then probabilities are
@@ -290,8 +277,6 @@ struct FwdDirectLayout {
   static constexpr int TOTAL_ELEMS = (STAGE_ELEMS > PATCH_ELEMS) ? STAGE_ELEMS : PATCH_ELEMS;
 };
 
-// s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt fields left at their maxima).
-__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
 
 template <typename T, int DP, int BKV>
@@ -304,7 +289,6 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
   __shared__ __attribute__((aligned(1024))) short smem[L::TOTAL_ELEMS];
-  FA2_STAMP(0);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -537,8 +521,6 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
       }
     }
   };
-
-  FA2_STAMP(1);
   // End of a tile: every wave is done with V_t and the K fragments of tile t+1 are in flight or
   // in registers; K_{t+2} and V_{t+1} (issued during this tile) have landed.  Then the fragment
   // pointers advance to K tile t+2 and V tile t+1 (stages are used round-robin).
@@ -571,8 +553,6 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
     step(2 * t + 1, std::integral_constant<int, 1>{}, std::false_type{});
     end_tile(t);
   }
-
-  FA2_STAMP(2);
   const float l_tot = sum_over_halves(l_run);
   const float inv_l = 1.f / l_tot;
   if (h == 0 && q0w + c < p.seqlen_q) LSE[q0w + c] = m_ref * p.scale + __logf(l_tot);
@@ -583,7 +563,6 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(oacc, inv_l, patch, O + (int64_t)q0w * p.o.stride_seq,
                               p.o.stride_seq, p.seqlen_q - q0w, DP, true);
-  FA2_STAMP(3);
 }
 
 }  // namespace fa2

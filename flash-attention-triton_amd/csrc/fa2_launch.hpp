@@ -1,0 +1,38 @@
+// Kernel launchers, one translation unit per kernel family so that the library builds in parallel.
+// `dp` is the padded head dimension of the table row in use (32, 64, 96, 128, 192 or 256); the
+// launchers pick the LDS-direct fast kernel when the tensors allow it and the generic one otherwise.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "fa2_params.hpp"
+
+namespace fa2 {
+
+// Which kernel a launcher picked (reported to callers that label measurements).
+enum KernelPath { kPathGeneric = 0, kPathDirect = 1 };
+
+// The fast kernels need the exact padded head dimension, 16-byte aligned rows and row offsets
+// inside a tile that fit 32 bits.
+inline bool direct_stride_ok(const Tensor4 &t) { return t.stride_seq < (int64_t(1) << 24); }
+inline bool direct_headdim(int dp, int headdim) {
+  return headdim == dp && (dp == 32 || dp == 64 || dp == 128);
+}
+inline bool fwd_direct_ok(int dp, const FwdParams &p) {
+  return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
+}
+inline bool dq_direct_ok(int dp, const BwdParams &p) {
+  return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
+}
+inline bool dkdv_direct_ok(int dp, const BwdParams &p) {
+  return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.q) && direct_stride_ok(p.d_o);
+}
+
+// bf16 != 0 selects the bf16 kernels, otherwise fp16.
+void launch_fwd(bool bf16, int dp, const FwdParams &p, dim3 grid, hipStream_t s);
+void launch_preprocess(bool bf16, const PreParams &p, dim3 grid, hipStream_t s);
+// fuse_delta: the fast dQ kernel also forms delta from O and dO (dq_direct_ok must hold).
+void launch_dq(bool bf16, int dp, const BwdParams &p, dim3 grid, bool fuse_delta, hipStream_t s);
+void launch_dkdv(bool bf16, int dp, const BwdParams &p, dim3 grid, hipStream_t s);
+
+}  // namespace fa2
