@@ -33,6 +33,8 @@ namespace fa2 {
 // formed against the stale maximum and may reach 2^kRescaleSlack, which fp32 sums and bf16/fp16
 // operands hold without loss.  The final division by the row sum removes the common factor.
 constexpr float kRescaleSlack = 8.0f;
+// The fast forward kernel tests a lane's sum of sixteen new probabilities instead of their maximum.
+constexpr float kSumTrigger = 1024.0f;
 
 template <int DP, int BKV>
 struct FwdLayout {
@@ -413,7 +415,10 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
     m_ref = row_max(sc);  // finite: every query row sees key 0
     const float mc = m_ref * scale_log2;
 #pragma unroll
-    for (int i = 0; i < 16; i++) e[i] = fast_exp2(sc[i] * scale_log2 - mc);
+    for (int i = 0; i < 16; i++) {
+      e[i] = fast_exp2(sc[i] * scale_log2 - mc);
+      l_run += e[i];
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) ring[ks] = k_frag(1, ks);
     // From here on kcur addresses K tile 1 (the tile after the current one).
@@ -470,12 +475,9 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
       for (int u = 0; u < 8 / KS; u++) {
         const int i = (8 / KS) * ks + u;  // probability pair (2i, 2i+1) of the 32 in the block
         w[i / 4][i % 4] = Elem<T>::pack2(e[2 * i], e[2 * i + 1]);
-        l_run += e[2 * i];
-        l_run += e[2 * i + 1];
       }
       // Pin the arithmetic to this unit: without a use here the optimiser sinks it next to the
       // MFMAs that consume it.
-      asm volatile("" : "+v"(l_run));
       if (ks == KS / 2 - 1) asm volatile("" : "+v"(w[0]));
       if (ks == KS - 1) asm volatile("" : "+v"(w[1]));
       __builtin_amdgcn_sched_barrier(0);
@@ -483,7 +485,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
     if (j + 1 >= n_full) apply_mask(sc, (j + 1) * BLK);
     const s16x8 pf[2] = {__builtin_bit_cast(s16x8, w[0]), __builtin_bit_cast(s16x8, w[1])};
     const float mc = m_ref * scale_log2;
-    float mloc = fmaxf(sc[0], sc[1]);
+    float lsum[2] = {0.f, 0.f};  // this lane's sum of the new probabilities, in two chains
 #pragma unroll
     for (int ks2 = 0; ks2 < 2; ks2++) {
 #pragma unroll
@@ -495,19 +497,22 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
 #pragma unroll
         for (int u = 0; u < 16 / KS; u++) {
           const int i = (16 / KS) * slot + u;
-          if (i >= 2) mloc = fmaxf(mloc, sc[i]);
           e[i] = fast_exp2(sc[i] * scale_log2 - mc);
+          lsum[i & 1] += e[i];
         }
-        asm volatile("" : "+v"(mloc));
+        asm volatile("" : "+v"(lsum[0]), "+v"(lsum[1]));
         asm volatile("" : "+v"(e));
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    mloc = max_over_halves(mloc);
     if (j + 1 < n_mine) {
-      const bool grow = (mloc - m_ref) * scale_log2 > kRescaleSlack;
+      // No maximum is taken on this path: a lane's sum of sixteen probabilities bounds each of
+      // them, so a sum above kSumTrigger (or one that overflowed to +inf) is what sends the wave
+      // to the rescale below.
+      float lblk = lsum[0] + lsum[1];
+      const bool grow = !(lblk <= kSumTrigger);
       if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-        const float m_new = fmaxf(m_ref, mloc);
+        const float m_new = fmaxf(m_ref, row_max(sc));
         const float alpha = fast_exp2((m_ref - m_new) * scale_log2);
         m_ref = m_new;
         l_run *= alpha;
@@ -516,11 +521,17 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
 #pragma unroll
           for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
         const float mc2 = m_new * scale_log2;
+        lblk = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; i++) e[i] = fast_exp2(sc[i] * scale_log2 - mc2);
+        for (int i = 0; i < 16; i++) {
+          e[i] = fast_exp2(sc[i] * scale_log2 - mc2);
+          lblk += e[i];
+        }
       }
+      l_run += lblk;
     }
   };
+
   // End of a tile: every wave is done with V_t and the K fragments of tile t+1 are in flight or
   // in registers; K_{t+2} and V_{t+1} (issued during this tile) have landed.  Then the fragment
   // pointers advance to K tile t+2 and V tile t+1 (stages are used round-robin).

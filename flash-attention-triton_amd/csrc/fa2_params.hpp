@@ -5,6 +5,9 @@
 
 namespace fa2 {
 
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
 // One (batch, nheads, seqlen, headdim) tensor: base pointer and strides in elements.
 struct Tensor4 {
   void *ptr;
