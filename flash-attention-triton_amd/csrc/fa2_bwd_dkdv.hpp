@@ -351,7 +351,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     float *sl = reinterpret_cast<float *>(smem + (t % L::STAGES) * L::STAGE_ELEMS + 2 * L::TILE_ELEMS);
     if (tid < BQ) {
       sl[tid] = lse_reg;
-      sl[BQ + tid] = delta_reg;
+      sl[BQ + tid] = -delta_reg;  // negated: it is the accumulator the dP MFMAs start from
     }
   };
   // Prologue: every global load of the first three tiles and of this wave's K and V rows is
@@ -456,7 +456,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 
     // ---- S = Q K^T (ring: Q rows -> dO^T); statistics of the 16 rows this lane holds ---------
     f32x16 s, dp;
-    f32x4 l4[4], d4[4];
+    f32x4 l4[4], d4[4];  // d4: minus delta of the rows this lane holds
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       if (ks == 0) VgprMfma<T>::first(s, ring[ks], kf[ks]);
@@ -482,8 +482,12 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     f32x16 pr;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      if (ks == 0) VgprMfma<T>::first(dp, ringb[ks], vf[ks]);
-      else VgprMfma<T>::next(dp, ringb[ks], vf[ks]);
+      // The chain starts from -delta, so that dS = P * dP needs no subtraction.
+      if (ks == 0)
+        dp = __builtin_shufflevector(__builtin_shufflevector(d4[0], d4[1], 0, 1, 2, 3, 4, 5, 6, 7),
+                                     __builtin_shufflevector(d4[2], d4[3], 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2,
+                                     3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+      VgprMfma<T>::next(dp, ringb[ks], vf[ks]);
       spread_load(KS + ks);
       {
         s16x4 a0 = lds_read_tr(qlo[ks % DB] + QOFF + 16 * (ks / DB) * DP);
@@ -518,7 +522,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 #pragma unroll
       for (int u = 0; u < 16 / KS; u++) {
         const int i = (16 / KS) * ks + u;
-        ds[i] = pr[i] * (dp[i] - d4[i >> 2][i & 3]);
+        ds[i] = pr[i] * dp[i];
       }
       asm volatile("" : "+v"(ds));
       __builtin_amdgcn_sched_barrier(0);
