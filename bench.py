@@ -30,18 +30,119 @@ sys.path.insert(0, str(ROOT))
 # Published dense peaks of MI355X.
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}
 CALIBRATION_BYTES = 256 << 20
-# HBM bytes per launch on workload C3 (bf16), read off rocprofv3's FETCH_SIZE / WRITE_SIZE counters
-# and scaled by what the same counters read for the --traffic-calibration copy (x2.000 / x1.000);
-# the summary sits in profiles/fwd_bwd_kernels_c3_bf16_hbm_traffic.txt.  Counters cannot be read
-# from inside the process, so other workloads report null.
-MEASURED_TRAFFIC_BYTES = {
-    ("C3", "fwd"): 776.7e6,
-    ("C3", "bwd_dkdv"): 878.5e6,
-    ("C3", "bwd_dq"): 842.2e6,
-    ("C3", "bwd_preprocess"): 135.3e6,
-}
+# HBM bytes per launch come from rocprofv3's FETCH_SIZE / WRITE_SIZE counters (counters cannot be
+# read from inside the process): the tracked summary below lists them per kernel for workload C3,
+# together with a hash of the kernel sources it was measured on.  Other workloads, or sources that
+# have changed since, report null.
+TRAFFIC_PROFILE = ROOT / "profiles" / "fwd_bwd_kernels_c3_bf16_hbm_traffic.txt"
+KERNEL_SOURCES = ROOT / "flash-attention-triton_amd" / "csrc"
 PEAK_HBM_GBS = 8000.0
 METRIC = "causal attn TFLOP/s fwd & fwd+bwd (bf16, D=128) and % of MFMA peak, 1 GPU"
+
+
+def kernel_sources_hash() -> str:
+    """sha256 over the kernel sources (names and contents), the stamp the traffic summary carries."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for path in sorted(KERNEL_SOURCES.glob("*.h*")):
+        h.update(path.name.encode())
+        h.update(path.read_bytes())
+    return h.hexdigest()[:16]
+
+
+def _measured_traffic(workload: str) -> tuple[dict, str]:
+    """{leg: bytes per launch} from the tracked counter summary, and a note saying why it is empty."""
+    if workload != "C3":
+        return {}, "the counter summary covers workload C3 only"
+    if not TRAFFIC_PROFILE.exists():
+        return {}, "no counter summary in profiles/"
+    stamp, rows = None, {}
+    for line in TRAFFIC_PROFILE.read_text().splitlines():
+        if line.startswith("kernel-sources-sha256:"):
+            stamp = line.split(":", 1)[1].strip()
+        if line.startswith("traffic-bytes "):
+            _, leg, value = line.split()
+            rows[leg] = float(value)
+    if stamp != kernel_sources_hash():
+        return {}, f"kernel sources changed since the counter summary was taken (summary {stamp}, now {kernel_sources_hash()})"
+    return rows, "profiles/" + TRAFFIC_PROFILE.name
+
+
+class ClockSampler:
+    """Samples the shader clock the driver reports (sysfs pp_dpm_sclk, the level marked '*') from
+    a background thread while a timed region runs."""
+
+    def __init__(self, period_s: float = 0.002):
+        import glob
+        import threading
+
+        files = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+        self.path = files[0] if files else None
+        self.period = period_s
+        self.samples: list[float] = []
+        self._stop = threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    def _read(self):
+        try:
+            with open(self.path) as f:
+                for line in f:
+                    if "*" in line:
+                        return float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+        except (OSError, ValueError, IndexError):
+            return None
+        return None
+
+    def _run(self):
+        while not self._stop.is_set():
+            v = self._read()
+            if v is not None:
+                self.samples.append(v)
+            self._stop.wait(self.period)
+
+    def __enter__(self):
+        if self.path:
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        if self.path:
+            self._thread.join()
+        return False
+
+    def summary(self):
+        if not self.samples:
+            return None
+        return {"samples": len(self.samples), "min": min(self.samples), "max": max(self.samples),
+                "mean": sum(self.samples) / len(self.samples)}
+
+
+def _device_clock_mhz(props) -> float:
+    """Maximum shader clock: torch's property when it is filled in, else hipDeviceAttributeClockRate."""
+    khz = getattr(props, "clock_rate", 0)
+    if not khz:
+        import ctypes
+
+        try:
+            hip = ctypes.CDLL("libamdhip64.so")
+            value = ctypes.c_int(0)
+            if hip.hipDeviceGetAttribute(ctypes.byref(value), 5, 0) == 0:  # hipDeviceAttributeClockRate, kHz
+                khz = value.value
+        except OSError:
+            khz = 0
+    return khz / 1e3
+
+
+def _cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def _load_package():
@@ -145,8 +246,8 @@ def _cpu_baseline(w, workloads, heads: int):
     ``heads`` (batch, head) slices of the same seeded workload, forward + backward."""
     from oracle import naive_attention as oracle
 
-    threads = os.cpu_count() or 1
-    threads = min(threads, 16)
+    # A one-GPU box's share of the host is 16 cores whatever os.cpu_count() shows there.
+    threads = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
     q, k, v, d_o = workloads.make_inputs(w, "cpu", heads=heads)
     t0 = time.perf_counter()
@@ -157,6 +258,8 @@ def _cpu_baseline(w, workloads, heads: int):
         "value": flops / dt / 1e12,
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
+        "os_cpu_count": os.cpu_count(),
+        "cpu_model": _cpu_model(),
         "kind": "port",
         "sample": f"{heads} of {w.batch * w.nheads} (batch, head) slices of {w.name}, fp32 forward+backward "
                   f"through torch autograd, {dt:.2f} s",
@@ -168,8 +271,12 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=50,
-                    help="untimed steps first; the GPU clocks need some tens of milliseconds of load to settle")
+    ap.add_argument("--warmup", type=int, default=50, help="untimed steps right before the timed ones")
+    ap.add_argument("--settle-ms", type=float, default=400.0,
+                    help="before the warm-up steps, run untimed steps for this long: an idle GPU sits at "
+                         "~100 MHz and its clocks and power controller need some hundreds of milliseconds of "
+                         "load to reach the steady state a training job runs in (the first 20 steps after 5 "
+                         "warm-up steps measure 5-6 %% slower than steady state)")
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--deterministic", action="store_true", help="time the deterministic backward in the step")
     ap.add_argument("--cpu-heads", type=int, default=64, help="(batch, head) slices in the CPU baseline sample")
@@ -208,23 +315,34 @@ def main() -> int:
         with torch.no_grad():
             return pkg.flash_attention_v2(q, k, v, scale, det)
 
+    def settle(fn):
+        t_end = time.perf_counter() + args.settle_ms * 1e-3
+        while time.perf_counter() < t_end:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+
+    settle(step)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    step_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    with ClockSampler() as step_clock:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        step_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    settle(fwd_only)
     for _ in range(max(args.warmup, 1)):
         fwd_only()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        fwd_only()
-    torch.cuda.synchronize()
-    fwd_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    with ClockSampler() as fwd_clock:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fwd_only()
+        torch.cuda.synchronize()
+        fwd_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
     dtype_name = "bf16" if w.dtype == torch.bfloat16 else "f16"
     peak = PEAK_TFLOPS[dtype_name]
@@ -237,18 +355,25 @@ def main() -> int:
     # FLOPs per launch, counted in causal GEMMs of fwd_flops / 2 each: the forward kernel owns 2
     # (S, PV), the dK/dV kernel 4 (S, dP, dV, dK), the dQ kernel 3 (S, dP, dQ).  The whole backward
     # is priced at the conventional 5 (2.5 x forward) although the two kernels execute 7.
+    # The LDS-direct kernels run when the table row has them and the head dimension needs no
+    # padding (the bench tensors are contiguous and 16-byte aligned); otherwise the generic ones.
+    fa2 = importlib.import_module("flash-attention-triton_amd.flash_attention_2")
+    row_id = capi.load().fa2_pick_config(fa2._COMPUTE_DTYPES[w.dtype], w.headdim, w.seqlen, w.seqlen, int(det))
+    row = capi.config_table()[row_id]
+    kind = "direct_kernel" if row["lds_direct"] and row["headdim_padded"] == w.headdim else "kernel"
     kernels = {
-        "fwd": ("fwd_direct_kernel (fa2_fwd)", 1.0 * w.fwd_flops),
-        "bwd_dkdv": ("bwd_dkdv_direct_kernel (fa2_bwd, dK/dV half)", 2.0 * w.fwd_flops),
-        "bwd_dq": ("bwd_dq_direct_kernel (fa2_bwd, dQ half)", 1.5 * w.fwd_flops),
+        "fwd": (f"fwd_{kind} (fa2_fwd)", 1.0 * w.fwd_flops),
+        "bwd_dkdv": (f"bwd_dkdv_{kind} (fa2_bwd, dK/dV half)", 2.0 * w.fwd_flops),
+        "bwd_dq": (f"bwd_dq_{kind} (fa2_bwd, dQ half)", 1.5 * w.fwd_flops),
     }
     dominant = max(kernels, key=lambda name: leg_ms[name])
+    traffic, traffic_source = _measured_traffic(w.name)
 
     def mfma_roofline(name):
         label, flops = kernels[name]
         achieved = flops / (leg_ms[name] * 1e-3) / 1e12
         return {"kernel": label, "bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, name)),
+                "frac": achieved / peak, "traffic": traffic.get(name), "traffic_source": traffic_source,
                 "flops_per_launch": flops,
                 "avg_launch_ms": leg_ms[name]}
 
@@ -260,7 +385,7 @@ def main() -> int:
         "kernel": "fa2_bwd_preprocess (bwd_preprocess_kernel)", "bound": "hbm",
         "achieved": pre_bytes / (leg_ms["bwd_preprocess"] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
         "frac": pre_bytes / (leg_ms["bwd_preprocess"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
-        "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, "bwd_preprocess")), "bytes_per_launch": pre_bytes,
+        "traffic": traffic.get("bwd_preprocess"), "bytes_per_launch": pre_bytes,
         "avg_launch_ms": leg_ms["bwd_preprocess"],
     }
 
@@ -291,7 +416,10 @@ def main() -> int:
         "peak_tflops": peak,
         "device": {"name": props.name, "arch": getattr(props, "gcnArchName", ""),
                    "compute_units": props.multi_processor_count,
-                   "clock_mhz": getattr(props, "clock_rate", 0) / 1e3},
+                   "clock_mhz": _device_clock_mhz(props),
+                   "sclk_mhz_during_steps": step_clock.summary(),
+                   "sclk_mhz_during_fwd": fwd_clock.summary()},
+        "settle_ms": args.settle_ms,
         "roofline": roofline,
         "roofline_fwd": mfma_roofline("fwd"),
         "roofline_bwd_dkdv": mfma_roofline("bwd_dkdv"),
@@ -300,6 +428,7 @@ def main() -> int:
         "bwd_frac_of_peak": bwd_tflops / peak,
         "roofline_bwd_preprocess": pre_roofline,
         "kernel_ms": leg_ms,
+        "table_row": row,
     }
     if args.traffic_calibration:
         src = torch.ones(CALIBRATION_BYTES // 4, device=dev, dtype=torch.float32)

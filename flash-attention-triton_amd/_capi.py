@@ -12,7 +12,7 @@ import pathlib
 import threading
 
 LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "csrc" / "libfa2_gfx950.so"
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 FA2_DTYPE_F16 = 0
 FA2_DTYPE_BF16 = 1
@@ -29,10 +29,37 @@ class ConfigInfo(ctypes.Structure):
         "id", "headdim_padded",
         "fwd_block_q", "fwd_block_kv", "fwd_waves",
         "bwd_block_q", "bwd_block_kv", "bwd_waves",
-        "dq_block_q", "dq_block_kv", "dq_waves")]
+        "dq_block_q", "dq_block_kv", "dq_waves",
+        "lds_direct", "fwd_wg_per_cu", "dq_wg_per_cu", "dkdv_wg_per_cu",
+        "lds_stages", "dkdv_passes", "head_group")]
 
     def as_dict(self) -> dict:
         return {name: getattr(self, name) for name, _ in self._fields_}
+
+
+class Tensor(ctypes.Structure):
+    """Mirror of ``fa2_tensor``: device pointer and the batch, head and sequence strides in elements."""
+
+    _fields_ = [("ptr", _p), ("stride_batch", _i64), ("stride_head", _i64), ("stride_seq", _i64)]
+
+
+class FwdArgs(ctypes.Structure):
+    """Mirror of ``fa2_fwd_args``."""
+
+    _fields_ = [("q", Tensor), ("k", Tensor), ("v", Tensor), ("o", Tensor), ("lse", _p),
+                ("batch", _i), ("nheads", _i), ("seqlen_q", _i), ("seqlen_k", _i), ("headdim", _i),
+                ("seqlen_q_rounded", _i), ("softmax_scale", _f), ("dtype", _i), ("config_id", _i)]
+
+
+class BwdArgs(ctypes.Structure):
+    """Mirror of ``fa2_bwd_args``."""
+
+    _fields_ = [("q", Tensor), ("k", Tensor), ("v", Tensor), ("o", Tensor), ("d_o", Tensor),
+                ("dq", Tensor), ("dk", Tensor), ("dv", Tensor), ("lse", _p), ("delta", _p),
+                ("workspace", _p),
+                ("batch", _i), ("nheads", _i), ("seqlen_q", _i), ("seqlen_k", _i), ("headdim", _i),
+                ("seqlen_q_rounded", _i), ("softmax_scale", _f), ("dtype", _i), ("deterministic", _i),
+                ("config_id", _i)]
 
 
 # Every symbol include/fa2_gfx950.h declares, with its ctypes signature.
@@ -48,6 +75,8 @@ SIGNATURES = {
     "fa2_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 7),
     "fa2_bwd": (_i, [_p] * 10 + [_i] * 6 + [_i64] * 21 + [_f, _i, _i, _i, _p]),
     "fa2_bwd_fused": (_i, [_p] * 11 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p]),
+    "fa2_fwd_packed": (_i, [ctypes.POINTER(FwdArgs), _p]),
+    "fa2_bwd_packed": (_i, [ctypes.POINTER(BwdArgs), _p]),
 }
 
 _lib = None

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, 1) void bwd_dkdv_kernel(const BwdPa
   // Key tile 0 has the longest query range: issue tiles in ascending order (heaviest first).
   const int BH = p.batch * p.nheads;
   int bh, kt;  // key tile 0 has the longest query range: rank == key tile
-  map_workgroup(blockIdx.x, BH, p.n_tiles, bh, kt);
+  map_workgroup(blockIdx.x, BH, p.n_tiles, p.head_group, bh, kt);
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int kv0 = kt * kDkvBlockKV;
   const int kv0w = kv0 + 32 * wave;
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   // Key tile 0 has the longest query range: issue tiles in ascending order (heaviest first).
   const int BH = p.batch * p.nheads;
   int bh, kt;  // key tile 0 has the longest query range: rank == key tile
-  map_workgroup(blockIdx.x, BH, p.n_tiles, bh, kt);
+  map_workgroup(blockIdx.x, BH, p.n_tiles, p.head_group, bh, kt);
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int kv0 = kt * kDkvBlockKV;
   const int kv0w = kv0 + 32 * wave;

@@ -35,8 +35,10 @@ template <typename T>
 __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const PreParams p) {
   const int tid = threadIdx.x;
   const int sub = tid & 15;
-  const int row = blockIdx.x * 16 + (tid >> 4);
-  const int bh = blockIdx.y;
+  // One-dimensional grid: row tiles of one (batch, head) pair are consecutive workgroups.
+  const int tiles = (p.seqlen_q_rounded + 15) / 16;
+  const int bh = blockIdx.x / tiles;
+  const int row = (blockIdx.x - bh * tiles) * 16 + (tid >> 4);
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const bool vec = p.vec != 0;
   float acc = 0.f;
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(64 * kDqWaves, (DP <= 96 ? 2 : 1)) void bwd_dq_kern
 
   const int BH = p.batch * p.nheads;
   int bh, rank;
-  map_workgroup(blockIdx.x, BH, p.n_tiles, bh, rank);
+  map_workgroup(blockIdx.x, BH, p.n_tiles, p.head_group, bh, rank);
   const int qt = p.n_tiles - 1 - rank;  // the last query tile sees the most keys
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int q0 = qt * kDqBlockQ;
@@ -280,7 +282,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
 
   const int BH = p.batch * p.nheads;
   int bh, rank;
-  map_workgroup(blockIdx.x, BH, p.n_tiles, bh, rank);
+  map_workgroup(blockIdx.x, BH, p.n_tiles, p.head_group, bh, rank);
   const int qt = p.n_tiles - 1 - rank;  // the last query tile sees the most keys
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int q0 = qt * kDqBlockQ;

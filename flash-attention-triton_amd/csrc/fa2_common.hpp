@@ -206,20 +206,21 @@ __device__ __forceinline__ void store_transposed_acc(const f32x16 (&acc)[DP / 32
 
 // Workgroup index -> (batch*head, tile rank); rank 0 is the heaviest tile of a head.
 //
-// Heads are taken 64 at a time: all tiles of a group of 64 heads, heaviest first, before the next
+// Heads are taken `group` at a time: all tiles of a group of heads, heaviest first, before the next
 // group starts.  The tiles of one head re-read the same K/V (or Q/dO) rows, so they should run
 // close together in time; with the heads merely round-robin over the whole grid, a problem with
 // thousands of (batch, head) pairs would have as many different heads in flight as the chip has
 // workgroup slots, nothing would be shared in L2 and every tile would stream its operand from HBM.
-// Workgroups go to the 8 XCDs round-robin and 64 is a multiple of 8, so a head also stays on one
-// XCD (one L2).  Up to 64 heads the order is simply head = i % heads, rank = i / heads.
-constexpr int kHeadGroup = 64;
-__device__ __forceinline__ void map_workgroup(int i, int heads, int tiles_per_head, int &bh, int &rank) {
-  const int per_group = kHeadGroup * tiles_per_head;
+// Workgroups go to the 8 XCDs round-robin and `group` is a multiple of 8, so a head also stays on
+// one XCD (one L2), `group / 8` heads sharing that L2 at a time.  The group size comes from the
+// gfx950 table (per kernel and problem size).
+__device__ __forceinline__ void map_workgroup(int i, int heads, int tiles_per_head, int group, int &bh,
+                                              int &rank) {
+  const int per_group = group * tiles_per_head;
   const int g = i / per_group;
   const int r = i - g * per_group;
-  const int gsize = min(kHeadGroup, heads - g * kHeadGroup);  // the last group may be smaller
-  bh = g * kHeadGroup + r % gsize;
+  const int gsize = min(group, heads - g * group);  // the last group may be smaller
+  bh = g * group + r % gsize;
   rank = r / gsize;
 }
 

@@ -149,7 +149,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_kerne
   // query tiles are issued heaviest (longest key range) first.
   const int BH = p.batch * p.nheads;
   int bh, rank;
-  map_workgroup(blockIdx.x, BH, p.n_qtiles, bh, rank);
+  map_workgroup(blockIdx.x, BH, p.n_qtiles, p.head_group, bh, rank);
   const int qt = p.n_qtiles - 1 - rank;  // the last query tile sees the most keys
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int q0 = qt * kFwdBlockQ;
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
 
   const int BH = p.batch * p.nheads;
   int bh, rank;
-  map_workgroup(blockIdx.x, BH, p.n_qtiles, bh, rank);
+  map_workgroup(blockIdx.x, BH, p.n_qtiles, p.head_group, bh, rank);
   const int qt = p.n_qtiles - 1 - rank;  // the last query tile sees the most keys
   const int b = bh / p.nheads, hd = bh % p.nheads;
   const int q0 = qt * kFwdBlockQ;

@@ -32,6 +32,7 @@ struct FwdParams {
   float *lse;
   int batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded;
   int n_qtiles;
+  int head_group;  // (batch, head) pairs whose tiles are dispatched together (multiple of 8)
   float scale;       // softmax scale (natural units)
   float scale_log2;  // scale * log2(e)
   int vec;           // 16-byte global accesses are legal for every tensor
@@ -45,6 +46,7 @@ struct BwdParams {
   const float *delta;
   int batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded;
   int n_tiles;  // key tiles (dK/dV kernel) or query tiles (dQ kernel)
+  int head_group;  // (batch, head) pairs whose tiles are dispatched together (multiple of 8)
   float scale, scale_log2;
   int vec;
 };

@@ -20,6 +20,7 @@ Differences from the reference, all deliberate:
 from __future__ import annotations
 
 import math
+import threading
 
 import torch
 
@@ -39,12 +40,15 @@ def _strides3(t: torch.Tensor) -> tuple[int, int, int]:
 
 
 _RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+# The binding functions behind torch.cuda.current_device(): the public wrappers add a lazy-init
+# check per call, about a microsecond each, which shows at the smallest problem sizes.
+_RAW_DEVICE = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
 
 
 def _stream_handle() -> int:
     """hipStream_t of torch's current stream on the current device, as an integer."""
     if _RAW_STREAM is not None:  # same value as below without building a Stream object (~10 us)
-        return _RAW_STREAM(torch.cuda.current_device())
+        return _RAW_STREAM(_RAW_DEVICE())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -61,9 +65,21 @@ class _NoGuard:
 
 _NO_GUARD = _NoGuard()
 
+# Argument records of the packed entry points, kept per problem signature and per thread (a record
+# is filled in and handed to the library by one thread at a time).
+_FWD_ARGS: dict = {}
+_BWD_ARGS: dict = {}
+_MAX_RECORDS = 256
+
+
+def _remember(table: dict, key, value) -> None:
+    if len(table) >= _MAX_RECORDS:
+        table.clear()
+    table[key] = value
+
 
 def _device_guard(device: torch.device):
-    if device.index is None or device.index == torch.cuda.current_device():
+    if device.index is None or device.index == _RAW_DEVICE():
         return _NO_GUARD
     return torch.cuda.device(device)
 
@@ -110,15 +126,29 @@ def _flash_attention_forward(
     # through) is folded into the sign of Q, which is exact: (-Q) K^T * |s| == Q K^T * s.
     q_in, kernel_scale = (q, softmax_scale) if softmax_scale > 0 else (-q, -softmax_scale)
 
+    # One argument record per (shapes, strides, dtype, scale), kept between calls: only the five
+    # pointers change from call to call.
+    key = (q_in.shape, seqlen_k, q_in.stride(), k.stride(), v.stride(), output.stride(), q.dtype,
+           seqlen_q_rounded, kernel_scale, threading.get_ident())
+    args = _FWD_ARGS.get(key)
+    if args is None:
+        args = _capi.FwdArgs()
+        for name, t in (("q", q_in), ("k", k), ("v", v), ("o", output)):
+            rec = getattr(args, name)
+            rec.stride_batch, rec.stride_head, rec.stride_seq = _strides3(t)
+        args.batch, args.nheads, args.seqlen_q, args.seqlen_k = batch, nheads, seqlen_q, seqlen_k
+        args.headdim, args.seqlen_q_rounded = headdim, seqlen_q_rounded
+        args.softmax_scale, args.dtype = kernel_scale, _COMPUTE_DTYPES[q.dtype]
+        args.config_id = _capi.FA2_CONFIG_AUTO
+        _remember(_FWD_ARGS, key, args)
+    args.q.ptr, args.k.ptr, args.v.ptr = q_in.data_ptr(), k.data_ptr(), v.data_ptr()
+    args.o.ptr, args.lse = output.data_ptr(), lse.data_ptr()
+
     lib = _capi.load()
     with _device_guard(q.device):
-        status = lib.fa2_fwd(
-            q_in.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), lse.data_ptr(),
-            batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded,
-            *_strides3(q_in), *_strides3(k), *_strides3(v), *_strides3(output),
-            kernel_scale, _COMPUTE_DTYPES[q.dtype], _capi.FA2_CONFIG_AUTO, _stream_handle(),
-        )
-    _capi.check(status, "fa2_fwd")
+        status = lib.fa2_fwd_packed(args, _stream_handle())
+    if status:
+        _capi.check(status, "fa2_fwd")
     return output, lse, softmax_scale  # softmax_scale could have been updated
 
 
@@ -161,7 +191,6 @@ def _flash_attention_backward(
     delta = torch.empty_like(lse)
     softmax_scale = softmax_scale or 1.0 / math.sqrt(headdim)
     deterministic = 1 if kernels_config.deterministic else 0
-    dtype = _COMPUTE_DTYPES[q.dtype]
 
     # Negative scale: run on -Q with |scale| (see the forward launcher); dK and dV are unchanged
     # and dQ comes out with the opposite sign.
@@ -169,24 +198,39 @@ def _flash_attention_backward(
     if negated:
         q, softmax_scale = -q, -softmax_scale
 
+    # Both launches of the reference launcher (preprocess, then the main kernel) in one call:
+    # with `o` in the record the library forms delta on the way.  Every tensor is contiguous here
+    # (asserted above), so shapes, dtype, scale and mode identify the record; the workspace size
+    # is asked once per record (it is 0: dQ is written directly).
+    key = (q.shape, seqlen_k, q.dtype, softmax_scale, deterministic, threading.get_ident())
+    cached = _BWD_ARGS.get(key)
+    if cached is None:
+        args = _capi.BwdArgs()
+        for name, t in (("q", q), ("k", k), ("v", v), ("o", output), ("d_o", d_output), ("dq", dq),
+                        ("dk", dk), ("dv", dv)):
+            rec = getattr(args, name)
+            rec.stride_batch, rec.stride_head, rec.stride_seq = _strides3(t)
+        args.batch, args.nheads, args.seqlen_q, args.seqlen_k = batch, nheads, seqlen_q, seqlen_k
+        args.headdim, args.seqlen_q_rounded = headdim, seqlen_q_rounded
+        args.softmax_scale, args.dtype = softmax_scale, _COMPUTE_DTYPES[q.dtype]
+        args.deterministic, args.config_id = deterministic, _capi.FA2_CONFIG_AUTO
+        ws_bytes = _capi.load().fa2_bwd_workspace_bytes(batch, nheads, seqlen_q, seqlen_k, headdim,
+                                                        deterministic, _capi.FA2_CONFIG_AUTO)
+        cached = (args, ws_bytes)
+        _remember(_BWD_ARGS, key, cached)
+    args, ws_bytes = cached
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+    args.q.ptr, args.k.ptr, args.v.ptr = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    args.o.ptr, args.d_o.ptr = output.data_ptr(), d_output.data_ptr()
+    args.dq.ptr, args.dk.ptr, args.dv.ptr = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    args.lse, args.delta = lse.data_ptr(), delta.data_ptr()
+    args.workspace = workspace.data_ptr() if workspace is not None else None
+
     lib = _capi.load()
     with _device_guard(q.device):
-        stream = _stream_handle()
-        ws_bytes = lib.fa2_bwd_workspace_bytes(batch, nheads, seqlen_q, seqlen_k, headdim,
-                                               deterministic, _capi.FA2_CONFIG_AUTO)
-        workspace = (torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None)
-        # Both launches of the reference launcher (preprocess, then the main kernel) in one call.
-        status = lib.fa2_bwd_fused(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), output.data_ptr(), d_output.data_ptr(),
-            lse.data_ptr(), delta.data_ptr(),
-            workspace.data_ptr() if workspace is not None else None,
-            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-            batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded,
-            *_strides3(q), *_strides3(k), *_strides3(v), *_strides3(output), *_strides3(d_output),
-            *_strides3(dq), *_strides3(dk), *_strides3(dv),
-            softmax_scale, dtype, deterministic, _capi.FA2_CONFIG_AUTO, stream,
-        )
-        _capi.check(status, "fa2_bwd_fused")
+        status = lib.fa2_bwd_packed(args, _stream_handle())
+    if status:
+        _capi.check(status, "fa2_bwd")
     if negated:
         dq.neg_()
 

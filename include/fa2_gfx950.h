@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define FA2_ABI_VERSION 1
+#define FA2_ABI_VERSION 2
 
 /* Largest head dimension the kernels accept (the table's `max_headdim`). */
 #define FA2_MAX_HEADDIM 256
@@ -72,10 +72,54 @@ typedef struct fa2_config_info {
   int bwd_block_q;    /* query rows per inner step, dK/dV kernel */
   int bwd_block_kv;   /* key rows per workgroup, dK/dV kernel */
   int bwd_waves;
-  int dq_block_q;     /* query rows per workgroup, dQ kernel (deterministic mode) */
+  int dq_block_q;     /* query rows per workgroup, dQ kernel */
   int dq_block_kv;
   int dq_waves;
+  int lds_direct;     /* 1: the row has LDS-direct kernels (global_load_lds into swizzled tiles) */
+  int fwd_wg_per_cu;  /* workgroups that share a CU (what registers and LDS leave room for) */
+  int dq_wg_per_cu;
+  int dkdv_wg_per_cu;
+  int lds_stages;     /* LDS stages of the streamed operand in the kernels of this row */
+  int dkdv_passes;    /* passes of the dK/dV kernel over the query tiles (2: half the columns each) */
+  int head_group;     /* (batch, head) pairs dispatched together; head_group / 8 share one XCD's L2 */
 } fa2_config_info;
+
+/* One (batch, nheads, seqlen, headdim) tensor: device pointer and strides in elements. */
+typedef struct fa2_tensor {
+  const void *ptr;
+  int64_t stride_batch, stride_head, stride_seq;
+} fa2_tensor;
+
+/*
+ * Arguments of fa2_fwd as one record (same meaning, field for field).  A caller that launches
+ * the same shapes repeatedly keeps the record and only swaps the pointers; a 27-argument call
+ * through a foreign-function interface costs more host time than the kernel launch it makes.
+ */
+typedef struct fa2_fwd_args {
+  fa2_tensor q, k, v, o; /* o is written */
+  float *lse;
+  int batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded;
+  float softmax_scale;
+  int dtype;
+  int config_id;
+} fa2_fwd_args;
+
+/*
+ * Arguments of the backward as one record.  o.ptr == NULL: `delta` is an input, as for fa2_bwd.
+ * o.ptr != NULL: `delta` is an output formed on the way, as for fa2_bwd_fused.  dq, dk and dv are
+ * written; dq.ptr == NULL or dk.ptr == dv.ptr == NULL skips that kernel (fa2_bwd's rule).
+ */
+typedef struct fa2_bwd_args {
+  fa2_tensor q, k, v, o, d_o, dq, dk, dv;
+  const float *lse;
+  float *delta;
+  void *workspace;
+  int batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded;
+  float softmax_scale;
+  int dtype;
+  int deterministic;
+  int config_id;
+} fa2_bwd_args;
 
 /* ABI version of the loaded library; equals FA2_ABI_VERSION of the header it was built from. */
 int fa2_abi_version(void);
@@ -114,6 +158,12 @@ int fa2_fwd(const void *q, const void *k, const void *v, void *o, float *lse,
             float softmax_scale, int dtype, int config_id, void *stream);
 
 /*
+ * fa2_fwd with its arguments in one record.  Same reference interface as fa2_fwd
+ * (flash_attention_2.py:61-144, _triton_kernels_v2.py:11-189).
+ */
+int fa2_fwd_packed(const fa2_fwd_args *args, void *stream);
+
+/*
  * Backward preprocess: delta[b,h,i] = sum_d O[b,h,i,d] * dO[b,h,i,d] in fp32.
  * Replaces _backward_preprocess_do_o_dot (_triton_kernels_v2.py:532-608; launched at
  * flash_attention_2.py:218-234).
@@ -125,8 +175,8 @@ int fa2_bwd_preprocess(const void *o, const void *d_o, float *delta,
                        int dtype, void *stream);
 
 /*
- * Bytes of fp32 workspace fa2_bwd needs for dQ accumulation (0 when the chosen mode writes dQ
- * directly).  Stands in for the reference's dq_accum allocation (flash_attention_2.py:196).
+ * Bytes of workspace the backward needs: 0, because dQ is written directly in both modes.
+ * Stands in for the reference's dq_accum allocation (flash_attention_2.py:196).
  */
 size_t fa2_bwd_workspace_bytes(int batch, int nheads, int seqlen_q, int seqlen_k, int headdim,
                                int deterministic, int config_id);
@@ -136,12 +186,16 @@ size_t fa2_bwd_workspace_bytes(int batch, int nheads, int seqlen_q, int seqlen_k
  * Replaces _flash_attention_backward's main launch, the dQ zero-fill pre-hook and the final
  * dq.copy_(dq_accum) (flash_attention_2.py:235-277, _configurators_v2.py:81-93,
  * _triton_kernels_v2.py:192-529).
- *   deterministic != 0: dQ is accumulated in a fixed order without atomics; results are
- *                       bit-identical from run to run.
- *   deterministic == 0: dQ may be accumulated with fp32 atomic adds into `workspace`
- *                       (sequence-parallel mode); low-order bits can differ between runs.
- * `workspace` must hold fa2_bwd_workspace_bytes(...) bytes (may be NULL when that is 0); the
- * library clears what it needs.
+ * Both values of `deterministic` run the same two kernels: a key-tile-parallel kernel for dK and
+ * dV and a query-tile-parallel kernel that accumulates dQ in registers in a fixed order and writes
+ * it once.  There are no atomics in either mode, so results are bit-identical from run to run in
+ * both (the reference's sequence-parallel mode, _triton_kernels_v2.py:336-339, allows run-to-run
+ * differences but does not require them).  The fp32 atomic-add formulation was measured on
+ * MI355X and rejected: the L2 retires about 1.35 TB/s of fp32 atomic adds whatever their
+ * locality, so the dQ contributions of a key-tile-parallel backward alone would take longer than
+ * the whole two-kernel backward.
+ * `workspace` is accepted for interface stability; fa2_bwd_workspace_bytes returns 0 and NULL is
+ * fine.
  * dK/dV and dQ are computed by two kernels launched back to back on `stream`.  A caller that
  * needs only part of the gradient (or wants to time one kernel) may pass dq == NULL to skip the
  * dQ kernel, or dk == dv == NULL to skip the dK/dV kernel; dk and dv are given or omitted
@@ -183,6 +237,12 @@ int fa2_bwd_fused(const void *q, const void *k, const void *v, const void *o, co
                   int64_t dk_stride_batch, int64_t dk_stride_head, int64_t dk_stride_seq,
                   int64_t dv_stride_batch, int64_t dv_stride_head, int64_t dv_stride_seq,
                   float softmax_scale, int dtype, int deterministic, int config_id, void *stream);
+
+/*
+ * The backward with its arguments in one record: fa2_bwd when args->o.ptr is NULL, fa2_bwd_fused
+ * otherwise.  Same reference interface (flash_attention_2.py:147-277).
+ */
+int fa2_bwd_packed(const fa2_bwd_args *args, void *stream);
 
 #ifdef __cplusplus
 }
