@@ -8,10 +8,13 @@ missing or reports an error, the caller gets an exception.
 from __future__ import annotations
 
 import ctypes
+import os
 import pathlib
 import threading
 
-LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "csrc" / "libfa2_gfx950.so"
+# The in-tree build; FA2_GFX950_LIBRARY names another build of the same ABI (e.g. one under test).
+LIBRARY_PATH = pathlib.Path(os.environ.get("FA2_GFX950_LIBRARY") or
+                            pathlib.Path(__file__).resolve().parent / "csrc" / "libfa2_gfx950.so")
 ABI_VERSION = 2
 
 FA2_DTYPE_F16 = 0

@@ -17,6 +17,11 @@ def build(force: bool = True) -> pathlib.Path:
     subprocess.run(cmd, check=True)
     if not LIBRARY.exists():
         raise RuntimeError(f"build did not produce {LIBRARY}")
+    # The measurement probes next to the kernels (stand-alone executables under probes/bin).
+    cmd = ["make", "-j2", "-C", str(CSRC / "probes")]
+    if force:
+        cmd.append("-B")
+    subprocess.run(cmd, check=True)
     return LIBRARY
 
 
