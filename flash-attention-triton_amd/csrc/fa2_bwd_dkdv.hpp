@@ -270,7 +270,8 @@ __device__ __forceinline__ void settle(f32x16 &d) { asm volatile("s_nop 11" : "+
 
 template <int DP, int BQ>
 struct DkvDirectLayout {
-  static constexpr int TILE_ELEMS = BQ * DP;
+  static constexpr int LP = lds_pitch(DP);  // LDS row pitch
+  static constexpr int TILE_ELEMS = BQ * LP;
   // One stage: Q tile, dO tile, then lse*log2e and delta as floats (2 shorts each).
   static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS + 4 * BQ;
   static constexpr int STAGES = 3;
@@ -282,7 +283,7 @@ struct DkvDirectLayout {
 template <typename T, int DP, int BQ>
 __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_direct_kernel(const BwdParams p) {
   using L = DkvDirectLayout<DP, BQ>;
-  constexpr int KS = DP / 16, DB = DP / 32;
+  constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
   constexpr int NTHREADS = 64 * kDkvWaves;
   static_assert(BQ == 64 && KS == 2 * DB, "schedule is written for 64-row query tiles of two blocks");
   static_assert(BQ <= NTHREADS, "one thread per row loads lse and delta");
@@ -390,7 +391,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   lds_cptr qnext[KS], qrow[KS], qlo[DB], qhi[DB];
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) {
-    qrow[ks] = lds0 + swz_off<DP>(c, 2 * ks + h);
+    qrow[ks] = lds0 + swz_off<LP>(c, 2 * ks + h);
     qnext[ks] = qrow[ks];
   }
   {
@@ -399,8 +400,8 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 #pragma unroll
     for (int db = 0; db < DB; db++) {
       const int chunk = 4 * db + 2 * g2 + ((i16 & 3) >> 1);
-      qlo[db] = lds0 + swz_off<DP>(rowlo, chunk) + sub;
-      qhi[db] = lds0 + swz_off<DP>(rowlo + 8, chunk) + sub;
+      qlo[db] = lds0 + swz_off<LP>(rowlo, chunk) + sub;
+      qhi[db] = lds0 + swz_off<LP>(rowlo + 8, chunk) + sub;
     }
   }
   const __attribute__((address_space(3))) float *stat =
@@ -432,7 +433,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   for (int ks = 0; ks < KS; ks++) ringb[ks] = lds_read_128(qrow[ks] + L::TILE_ELEMS);
 
   // One 32-row query block.  HALF selects the half-tile; MASKED switches the causal/row masks on.
-  // With SPREAD the block also issues the global->LDS loads of tile `lt`, one every fourth unit:
+  // With SPREAD the block also issues the global->LDS loads of tile `lt`, one every few units:
   // issued back to back by all waves after a barrier they queue up in the memory pipeline, and a
   // wave whose load cannot issue cannot issue its MFMAs either.
   auto block = [&](int qb, auto half_tag, auto masked_tag, auto spread_tag, int lt) {
@@ -440,17 +441,18 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     constexpr bool MASKED = decltype(masked_tag)::value;
     constexpr bool SPREAD = decltype(spread_tag)::value;
     constexpr int LOADS = TileLoader<DP, BQ, kDkvWaves>::LOADS;
-    static_assert(4 * KS == 8 * LOADS, "one load every fourth unit covers both tiles");
+    constexpr int EVERY = 4 * KS / (2 * LOADS);  // units between loads: both tiles' loads fit the block
+    static_assert(EVERY >= 1 && (2 * LOADS - 1) * EVERY < 4 * KS, "the block must have room for both tiles' loads");
     const unsigned ldst = lds_base + 2u * (unsigned)((lt % L::STAGES) * L::STAGE_ELEMS);
     const int lrow0 = q_begin + lt * BQ;
     auto spread_load = [&](int unit) {  // unit: 0 .. 4 KS - 1 over the four GEMMs
-      if (SPREAD && unit % 4 == 0) {
-        const int li = unit / 4;
+      if (SPREAD && unit % EVERY == 0 && unit / EVERY < 2 * LOADS) {
+        const int li = unit / EVERY;
         if (li < LOADS) qload.issue_one(lrow0, ldst, li);
         else gload.issue_one(lrow0, ldst + 2u * L::TILE_ELEMS, li - LOADS);
       }
     };
-    constexpr int QOFF = HALF * 32 * DP;          // Q rows of this block inside the tile
+    constexpr int QOFF = HALF * 32 * LP;          // Q rows of this block inside the tile
     constexpr int GOFF = QOFF + L::TILE_ELEMS;    // dO rows of this block
     typedef const __attribute__((address_space(3))) f32x4 *stat4_ptr;
 
@@ -463,8 +465,8 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       else VgprMfma<T>::next(s, ring[ks], kf[ks]);
       spread_load(ks);
       {
-        s16x4 a0 = lds_read_tr(qlo[ks % DB] + GOFF + 16 * (ks / DB) * DP);
-        s16x4 a1 = lds_read_tr(qhi[ks % DB] + GOFF + 16 * (ks / DB) * DP);
+        s16x4 a0 = lds_read_tr(qlo[ks % DB] + GOFF + 16 * (ks / DB) * LP);
+        s16x4 a1 = lds_read_tr(qhi[ks % DB] + GOFF + 16 * (ks / DB) * LP);
         ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
       constexpr int PER = (4 + KS - 1) / KS;  // row groups of four fetched per unit
@@ -490,14 +492,13 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       VgprMfma<T>::next(dp, ringb[ks], vf[ks]);
       spread_load(KS + ks);
       {
-        s16x4 a0 = lds_read_tr(qlo[ks % DB] + QOFF + 16 * (ks / DB) * DP);
-        s16x4 a1 = lds_read_tr(qhi[ks % DB] + QOFF + 16 * (ks / DB) * DP);
+        s16x4 a0 = lds_read_tr(qlo[ks % DB] + QOFF + 16 * (ks / DB) * LP);
+        s16x4 a1 = lds_read_tr(qhi[ks % DB] + QOFF + 16 * (ks / DB) * LP);
         ringb[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
       if (ks == 0) settle(s);  // after the S chain's last MFMA and before the first read of S
 #pragma unroll
-      for (int u = 0; u < 16 / KS; u++) {
-        const int i = (16 / KS) * ks + u;
+      for (int i = part(16, KS, ks); i < part(16, KS, ks + 1); i++) {
         float x = fast_exp2(s[i] * scale_log2 - l4[i >> 2][i & 3]);
         if (MASKED) {
           const int qr = qb + 8 * (i >> 2) + 4 * h + (i & 3);
@@ -517,13 +518,10 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     for (int ks = 0; ks < KS; ks++) {
       dvacc[ks % DB] = Elem<T>::mfma(ring[ks], pf[ks / DB], dvacc[ks % DB]);
       spread_load(2 * KS + ks);
-      ring[ks] = lds_read_128(qnext[ks] + (HALF == 0 ? 32 * DP : 0));
+      ring[ks] = lds_read_128(qnext[ks] + (HALF == 0 ? 32 * LP : 0));
       if (ks == 0) settle(dp);
 #pragma unroll
-      for (int u = 0; u < 16 / KS; u++) {
-        const int i = (16 / KS) * ks + u;
-        ds[i] = pr[i] * dp[i];
-      }
+      for (int i = part(16, KS, ks); i < part(16, KS, ks + 1); i++) ds[i] = pr[i] * dp[i];
       asm volatile("" : "+v"(ds));
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -535,7 +533,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     for (int ks = 0; ks < KS; ks++) {
       dkacc[ks % DB] = Elem<T>::mfma(ringb[ks], dsf[ks / DB], dkacc[ks % DB]);
       spread_load(3 * KS + ks);
-      ringb[ks] = lds_read_128(qnext[ks] + L::TILE_ELEMS + (HALF == 0 ? 32 * DP : 0));
+      ringb[ks] = lds_read_128(qnext[ks] + L::TILE_ELEMS + (HALF == 0 ? 32 * LP : 0));
       __builtin_amdgcn_sched_barrier(0);
     }
   };

@@ -12,6 +12,7 @@ void launch(int dp, const BwdParams &p, dim3 grid, hipStream_t s) {
     switch (dp) {
       case 32: hipLaunchKernelGGL((bwd_dkdv_direct_kernel<T, 32, kDkvBlockQ>), grid, block, 0, s, p); break;
       case 64: hipLaunchKernelGGL((bwd_dkdv_direct_kernel<T, 64, kDkvBlockQ>), grid, block, 0, s, p); break;
+      case 96: hipLaunchKernelGGL((bwd_dkdv_direct_kernel<T, 96, kDkvBlockQ>), grid, block, 0, s, p); break;
       default: hipLaunchKernelGGL((bwd_dkdv_direct_kernel<T, 128, kDkvBlockQ>), grid, block, 0, s, p); break;
     }
     return;

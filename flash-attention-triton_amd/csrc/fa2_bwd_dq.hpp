@@ -253,7 +253,8 @@ __global__ __launch_bounds__(64 * kDqWaves, (DP <= 96 ? 2 : 1)) void bwd_dq_kern
 // tile t+1, so that the K rows of the next tile are there when the last block of a tile fetches them.
 template <int DP, int BKV>
 struct DqDirectLayout {
-  static constexpr int TILE_ELEMS = BKV * DP;
+  static constexpr int LP = lds_pitch(DP);  // LDS row pitch
+  static constexpr int TILE_ELEMS = BKV * LP;
   static constexpr int K_STAGES = 3, V_STAGES = 2;
   static constexpr int K_BASE = 0;
   static constexpr int V_BASE = K_STAGES * TILE_ELEMS;
@@ -268,7 +269,7 @@ struct DqDirectLayout {
 template <typename T, int DP, int BKV, bool FUSE_DELTA>
 __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const BwdParams p) {
   using L = DqDirectLayout<DP, BKV>;
-  constexpr int KS = DP / 16, DB = DP / 32;
+  constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
   constexpr int BLK = 32;
   static_assert(BKV == 2 * BLK, "written for 64-row key tiles of two 32-row blocks");
 
@@ -358,8 +359,8 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   lds_cptr knext[KS], vrow[KS], klo[DB], khi[DB];
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) {
-    knext[ks] = lds0 + L::K_BASE + swz_off<DP>(c, 2 * ks + h);
-    vrow[ks] = lds0 + L::V_BASE + swz_off<DP>(c, 2 * ks + h);
+    knext[ks] = lds0 + L::K_BASE + swz_off<LP>(c, 2 * ks + h);
+    vrow[ks] = lds0 + L::V_BASE + swz_off<LP>(c, 2 * ks + h);
   }
   {
     const int rowlo = 4 * h + (i16 >> 2);
@@ -367,8 +368,8 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
 #pragma unroll
     for (int db = 0; db < DB; db++) {
       const int chunk = 4 * db + 2 * g2 + ((i16 & 3) >> 1);
-      klo[db] = lds0 + L::K_BASE + swz_off<DP>(rowlo, chunk) + sub;
-      khi[db] = lds0 + L::K_BASE + swz_off<DP>(rowlo + 8, chunk) + sub;
+      klo[db] = lds0 + L::K_BASE + swz_off<LP>(rowlo, chunk) + sub;
+      khi[db] = lds0 + L::K_BASE + swz_off<LP>(rowlo + 8, chunk) + sub;
     }
   }
 
@@ -408,12 +409,12 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
     }
     const unsigned kdst = lds_base + 2u * (unsigned)(L::K_BASE + (kt % L::K_STAGES) * L::TILE_ELEMS);
     const unsigned vdst = lds_base + 2u * (unsigned)(L::V_BASE + (vt % L::V_STAGES) * L::TILE_ELEMS);
-    constexpr int HOFF = HALF * BLK * DP;
+    constexpr int HOFF = HALF * BLK * LP;
     f32x16 s = zero, dp = zero;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       s = Elem<T>::mfma(ring[ks], qf[ks], s);
-      if (SPREAD && ks % LOAD_EVERY == 0) vload.issue_one(vt * BKV, vdst, ks / LOAD_EVERY);
+      if (SPREAD && ks % LOAD_EVERY == 0 && ks / LOAD_EVERY < LOADS) vload.issue_one(vt * BKV, vdst, ks / LOAD_EVERY);
       ring[ks] = lds_read_128(vrow[ks] + HOFF);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -421,15 +422,14 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       dp = Elem<T>::mfma(ring[ks], gf[ks], dp);
-      if (SPREAD && ks % LOAD_EVERY == 0) kload.issue_one(kt * BKV, kdst, ks / LOAD_EVERY);
+      if (SPREAD && ks % LOAD_EVERY == 0 && ks / LOAD_EVERY < LOADS) kload.issue_one(kt * BKV, kdst, ks / LOAD_EVERY);
       {
-        s16x4 a0 = lds_read_tr(klo[ks % DB] + HOFF + 16 * (ks / DB) * DP);
-        s16x4 a1 = lds_read_tr(khi[ks % DB] + HOFF + 16 * (ks / DB) * DP);
+        s16x4 a0 = lds_read_tr(klo[ks % DB] + HOFF + 16 * (ks / DB) * LP);
+        s16x4 a1 = lds_read_tr(khi[ks % DB] + HOFF + 16 * (ks / DB) * LP);
         ring[ks] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
 #pragma unroll
-      for (int u = 0; u < 16 / KS; u++) {
-        const int i = (16 / KS) * ks + u;
+      for (int i = part(16, KS, ks); i < part(16, KS, ks + 1); i++) {
         float pr = fast_exp2(s[i] * scale_log2 - lse2);
         if (need_mask) {
           const int kv = j * BLK + 8 * (i >> 2) + 4 * h + (i & 3);
@@ -451,13 +451,11 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
       constexpr int HALF_SLOTS = KS / 2;
       const int ks2 = slot / DB, db = slot % DB;
       dqacc[db] = Elem<T>::mfma(ring[slot], dsf[ks2], dqacc[db]);
-      ring[slot] = lds_read_128(knext[slot] + (HALF == 0 ? BLK * DP : 0));
+      ring[slot] = lds_read_128(knext[slot] + (HALF == 0 ? BLK * LP : 0));
       if (slot < HALF_SLOTS) {
 #pragma unroll
-        for (int u = 0; u < 8 / HALF_SLOTS; u++) {
-          const int i = (8 / HALF_SLOTS) * slot + u;
+        for (int i = part(8, HALF_SLOTS, slot); i < part(8, HALF_SLOTS, slot + 1); i++)
           hi[i] = s[8 + i] * (dp[8 + i] - delta);
-        }
         asm volatile("" : "+v"(hi));
         if (slot == HALF_SLOTS - 1) dsf[1] = Elem<T>::pack8(hi);
       }

@@ -10,6 +10,7 @@ void launch_direct(int dp, const BwdParams &p, dim3 grid, dim3 block, hipStream_
   switch (dp) {
     case 32: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 32, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
     case 64: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 64, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
+    case 96: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 96, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
     default: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 128, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
   }
 }

@@ -42,7 +42,7 @@ const fa2_config_info kTable[] = {
     // id DP  fwd:BQ       BKV        waves dK/dV:BQ   BKV       waves dQ:BQ    BKV      waves fast fwd/CU dq/CU dkdv/CU stages passes group
     {0, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 4, 3, 3, 1, kHeadGroup},
     {1, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 3, 2, 3, 1, kHeadGroup},
-    {2, 96, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 2, 2, 1, 2, 1, kHeadGroup},
+    {2, 96, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup},
     {3, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup},
     {4, 192, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 1, kHeadGroup},
     {5, 256, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 2, kHeadGroup},

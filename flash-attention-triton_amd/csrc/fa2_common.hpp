@@ -298,11 +298,23 @@ __device__ __forceinline__ void load_lds_16(const short *uniform_base, unsigned 
 // s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt fields left at their maxima).
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-// Streams ROWS x DP tiles of a (seqlen, headdim) matrix into swizzled LDS with LDS-direct loads.
-// All NW waves of the workgroup take part; each wave issues LOADS loads of 1 KiB per tile.
+// Row pitch, in elements, of the LDS tiles of the fast kernels for head dimension DP.  The swizzle
+// needs a power-of-two number of 16-byte chunks per row, so 96 columns live in rows of 128: the
+// last four chunk slots of a row are never loaded and never read.
+constexpr int lds_pitch(int dp) { return dp == 96 ? 128 : dp; }
+
+// Items [part(n, units, u), part(n, units, u + 1)) are unit u's share of n items spread as evenly
+// as integers allow over `units` units (equal shares when units divides n).
+constexpr int part(int n, int units, int u) { return n * u / units; }
+
+// Streams ROWS x DP tiles of a (seqlen, headdim) matrix into swizzled LDS (row pitch lds_pitch(DP))
+// with LDS-direct loads.  All NW waves of the workgroup take part; each wave issues LOADS loads of
+// 1 KiB of LDS per tile.  A lane owns one 16-byte slot of a row; lanes whose slot holds no data
+// (DP < pitch) are switched off for the load.
 template <int DP, int ROWS, int NW>
 struct TileLoader {
-  static constexpr int CPR = DP / 8;    // chunks per row
+  static constexpr int LP = lds_pitch(DP);
+  static constexpr int CPR = LP / 8;    // chunk slots per row
   static constexpr int RPL = 64 / CPR;  // rows per wave-load
   static constexpr int NL = ROWS / RPL; // wave-loads per tile
   static constexpr int LOADS = NL / NW; // per wave
@@ -310,7 +322,7 @@ struct TileLoader {
   // Multiples of NW*RPL rows keep the low four row bits the swizzle looks at, so a lane's
   // swizzled chunk does not depend on the load index.
   static_assert((NW * RPL) % 16 == 0, "swizzle must be independent of the load index");
-  static constexpr int TILE_ELEMS = ROWS * DP;
+  static constexpr int TILE_ELEMS = ROWS * LP;
 
   const short *base;  // first row of the matrix for this (batch, head)
   int64_t stride;     // row stride in elements
@@ -318,28 +330,29 @@ struct TileLoader {
   int row_in;         // this lane's row within the tile for load 0
   int chunk;          // this lane's global chunk index
   unsigned voff;      // byte offset of this lane inside a tile for load 0
+  bool active;        // this lane's slot holds data
 
   __device__ __forceinline__ TileLoader(const short *base_, int64_t stride_) : base(base_), stride(stride_) {
     const int lane = threadIdx.x & 63;
     wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     row_in = wave * RPL + lane / CPR;
-    chunk = (lane % CPR) ^ swz<DP>(row_in);
+    chunk = (lane % CPR) ^ swz<LP>(row_in);
+    active = LP == DP || chunk < DP / 8;
     voff = 2u * (unsigned)(row_in * (int)stride + chunk * 8);
   }
 
   // Rows [row0, row0 + ROWS), all inside the matrix -> tile at LDS byte address `lds`.
   __device__ __forceinline__ void issue(int row0, unsigned lds) const {
-    const short *tile = base + (int64_t)row0 * stride;
 #pragma unroll
-    for (int i = 0; i < LOADS; i++)
-      load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (unsigned)(i * NW + wave) * 1024u);
+    for (int i = 0; i < LOADS; i++) issue_one(row0, lds, i);
   }
 
   // Wave-load i (0 <= i < LOADS) of the same tile alone, for callers that spread a tile's loads
   // between other work.
   __device__ __forceinline__ void issue_one(int row0, unsigned lds, int i) const {
     const short *tile = base + (int64_t)row0 * stride;
-    load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (unsigned)(i * NW + wave) * 1024u);
+    if (LP == DP || active)
+      load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (unsigned)(i * NW + wave) * 1024u);
   }
 
   // Same, but rows at or beyond `nrows` are taken from row nrows - 1 (finite values that the
@@ -348,7 +361,8 @@ struct TileLoader {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
       const int r = min(row0 + i * NW * RPL + row_in, nrows - 1);
-      load_lds_16(base + (int64_t)r * stride + chunk * 8, lds + (unsigned)(i * NW + wave) * 1024u);
+      if (LP == DP || active)
+        load_lds_16(base + (int64_t)r * stride + chunk * 8, lds + (unsigned)(i * NW + wave) * 1024u);
     }
   }
 };

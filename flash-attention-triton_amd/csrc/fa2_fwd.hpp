@@ -270,7 +270,8 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_kerne
 // ------------------------------------------------------------------------------------------
 template <int DP, int BKV>
 struct FwdDirectLayout {
-  static constexpr int TILE_ELEMS = BKV * DP;
+  static constexpr int LP = lds_pitch(DP);  // LDS row pitch
+  static constexpr int TILE_ELEMS = BKV * LP;
   static constexpr int K_STAGES = 3, V_STAGES = 2;
   static constexpr int K_BASE = 0;
   static constexpr int V_BASE = K_STAGES * TILE_ELEMS;
@@ -284,7 +285,7 @@ struct FwdDirectLayout {
 template <typename T, int DP, int BKV>
 __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const FwdParams p) {
   using L = FwdDirectLayout<DP, BKV>;
-  constexpr int KS = DP / 16, DB = DP / 32;
+  constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
   constexpr int NTHREADS = 64 * kFwdWaves;
   constexpr int BLK = 32;  // keys per pipeline block
   static_assert(BKV == 2 * BLK && KS == 2 * DB, "schedule is written for 64-row tiles of two blocks");
@@ -354,23 +355,23 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   lds_cptr kcur[KS], vlo[DB], vhi[DB];
   const lds_cptr lds0 = to_lds(smem);
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) kcur[ks] = lds0 + L::K_BASE + swz_off<DP>(c, 2 * ks + h);
+  for (int ks = 0; ks < KS; ks++) kcur[ks] = lds0 + L::K_BASE + swz_off<LP>(c, 2 * ks + h);
   {
     const int rowlo = 4 * h + (i16 >> 2);
     const int sub = (i16 & 1) * 4;
 #pragma unroll
     for (int db = 0; db < DB; db++) {
       const int chunk = 4 * db + 2 * g2 + ((i16 & 3) >> 1);
-      vlo[db] = lds0 + L::V_BASE + swz_off<DP>(rowlo, chunk) + sub;
-      vhi[db] = lds0 + L::V_BASE + swz_off<DP>(rowlo + 8, chunk) + sub;
+      vlo[db] = lds0 + L::V_BASE + swz_off<LP>(rowlo, chunk) + sub;
+      vhi[db] = lds0 + L::V_BASE + swz_off<LP>(rowlo + 8, chunk) + sub;
     }
   }
   // K fragment ks of the half-tile `half` of the tile kcur points at.
-  auto k_frag = [&](int half, int ks) { return lds_read_128(kcur[ks] + half * BLK * DP); };
+  auto k_frag = [&](int half, int ks) { return lds_read_128(kcur[ks] + half * BLK * LP); };
   // V^T fragment (k-step ks2 in {0,1} of half-tile `half`, head-dim block db) of the tile vcur points at.
   auto v_frag = [&](int half, int ks2, int db) -> s16x8 {
-    s16x4 lo = lds_read_tr(vlo[db] + half * BLK * DP + 16 * ks2 * DP);
-    s16x4 hi = lds_read_tr(vhi[db] + half * BLK * DP + 16 * ks2 * DP);
+    s16x4 lo = lds_read_tr(vlo[db] + half * BLK * LP + 16 * ks2 * LP);
+    s16x4 hi = lds_read_tr(vhi[db] + half * BLK * LP + 16 * ks2 * LP);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
@@ -449,7 +450,8 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   // time between the units of tile t's first step.  Issued back to back by all waves at once they
   // queue up in the memory pipeline, and a wave whose load cannot issue cannot issue its MFMAs
   // either.
-  constexpr int LOAD_EVERY = KS / TileLoader<DP, BKV, kFwdWaves>::LOADS;
+  constexpr int LOADS = TileLoader<DP, BKV, kFwdWaves>::LOADS;
+  constexpr int LOAD_EVERY = KS / LOADS;
   auto step = [&](int j, auto half_tag, auto spread_tag) {
     constexpr int HALF = decltype(half_tag)::value;
     constexpr bool SPREAD = decltype(spread_tag)::value;
@@ -469,13 +471,11 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       sc = Elem<T>::mfma(ring[ks], qf[ks], sc);
-      if (SPREAD && ks % LOAD_EVERY == 0) vload.issue_one(vt * BKV, vdst, ks / LOAD_EVERY);
+      if (SPREAD && ks % LOAD_EVERY == 0 && ks / LOAD_EVERY < LOADS) vload.issue_one(vt * BKV, vdst, ks / LOAD_EVERY);
       ring[ks] = v_frag(HALF, ks / DB, ks % DB);
 #pragma unroll
-      for (int u = 0; u < 8 / KS; u++) {
-        const int i = (8 / KS) * ks + u;  // probability pair (2i, 2i+1) of the 32 in the block
+      for (int i = part(8, KS, ks); i < part(8, KS, ks + 1); i++)  // probability pair (2i, 2i+1) of the block
         w[i / 4][i % 4] = Elem<T>::pack2(e[2 * i], e[2 * i + 1]);
-      }
       // Pin the arithmetic to this unit: without a use here the optimiser sinks it next to the
       // MFMAs that consume it.
       if (ks == KS / 2 - 1) asm volatile("" : "+v"(w[0]));
@@ -492,11 +492,10 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
       for (int db = 0; db < DB; db++) {
         const int slot = ks2 * DB + db;
         oacc[db] = Elem<T>::mfma(ring[slot], pf[ks2], oacc[db]);
-        if (SPREAD && slot % LOAD_EVERY == 0) kload.issue_one(kt * BKV, kdst, slot / LOAD_EVERY);
+        if (SPREAD && slot % LOAD_EVERY == 0 && slot / LOAD_EVERY < LOADS) kload.issue_one(kt * BKV, kdst, slot / LOAD_EVERY);
         ring[slot] = k_frag(HALF, slot);
 #pragma unroll
-        for (int u = 0; u < 16 / KS; u++) {
-          const int i = (16 / KS) * slot + u;
+        for (int i = part(16, KS, slot); i < part(16, KS, slot + 1); i++) {
           e[i] = fast_exp2(sc[i] * scale_log2 - mc);
           lsum[i & 1] += e[i];
         }

@@ -24,6 +24,7 @@ void launch(int dp, const FwdParams &p, dim3 grid, hipStream_t s) {
     switch (dp) {
       case 32: hipLaunchKernelGGL((fwd_direct_kernel<T, 32, kFwdBlockKV>), grid, block, 0, s, p); break;
       case 64: hipLaunchKernelGGL((fwd_direct_kernel<T, 64, kFwdBlockKV>), grid, block, 0, s, p); break;
+      case 96: hipLaunchKernelGGL((fwd_direct_kernel<T, 96, kFwdBlockKV>), grid, block, 0, s, p); break;
       default: hipLaunchKernelGGL((fwd_direct_kernel<T, 128, kFwdBlockKV>), grid, block, 0, s, p); break;
     }
     return;

@@ -16,7 +16,7 @@ enum KernelPath { kPathGeneric = 0, kPathDirect = 1 };
 // inside a tile that fit 32 bits.
 inline bool direct_stride_ok(const Tensor4 &t) { return t.stride_seq < (int64_t(1) << 24); }
 inline bool direct_headdim(int dp, int headdim) {
-  return headdim == dp && (dp == 32 || dp == 64 || dp == 128);
+  return headdim == dp && (dp == 32 || dp == 64 || dp == 96 || dp == 128);
 }
 inline bool fwd_direct_ok(int dp, const FwdParams &p) {
   return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
