@@ -307,6 +307,13 @@ constexpr int lds_pitch(int dp) { return dp == 96 ? 128 : dp; }
 // as integers allow over `units` units (equal shares when units divides n).
 constexpr int part(int n, int units, int u) { return n * u / units; }
 
+// Workgroup barrier between two tiles of a streaming loop, without the "wait for every
+// outstanding LDS operation" the compiler puts in front of a barrier it can see.  The caller has
+// already waited for its LDS-direct loads (vmcnt); the LDS reads still in flight at this point
+// fetch fragments from a stage that nothing overwrites before the next barrier, so they may
+// complete after it.
+__device__ __forceinline__ void tile_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
 // Streams ROWS x DP tiles of a (seqlen, headdim) matrix into swizzled LDS (row pitch lds_pitch(DP))
 // with LDS-direct loads.  All NW waves of the workgroup take part; each wave issues LOADS loads of
 // 1 KiB of LDS per tile.  A lane owns one 16-byte slot of a row; lanes whose slot holds no data

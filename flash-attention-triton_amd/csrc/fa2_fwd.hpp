@@ -282,6 +282,14 @@ struct FwdDirectLayout {
 
 
 
+// Which half of a 64-row tile a step works on, and whether the step is known to lie well inside
+// the wave's key range (no block-count tests needed).
+template <int HALF, bool INNER>
+struct HalfTag {
+  static constexpr int value = HALF;
+  static constexpr bool inner = INNER;
+};
+
 template <typename T, int DP, int BKV>
 __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const FwdParams p) {
   using L = FwdDirectLayout<DP, BKV>;
@@ -455,7 +463,10 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   auto step = [&](int j, auto half_tag, auto spread_tag) {
     constexpr int HALF = decltype(half_tag)::value;
     constexpr bool SPREAD = decltype(spread_tag)::value;
-    if (j >= n_mine) {
+    // SPREAD steps and the step after them lie at least two tiles before the wave's diagonal:
+    // blocks j and j + 1 are always the wave's own there, and the tests below fold away.
+    constexpr bool INNER = decltype(spread_tag)::value || decltype(half_tag)::inner;
+    if (!INNER && j >= n_mine) {
       if (SPREAD) {  // not reached: the skipped blocks lie in the last two tiles, which load nothing
         issue_k(j / 2 + 2);
         issue_v(j / 2 + 1);
@@ -504,7 +515,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    if (j + 1 < n_mine) {
+    if (INNER || j + 1 < n_mine) {
       // No maximum is taken on this path: a lane's sum of sixteen probabilities bounds each of
       // them, so a sum above kSumTrigger (or one that overflowed to +inf) is what sends the wave
       // to the rescale below.
@@ -536,7 +547,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   // pointers advance to K tile t+2 and V tile t+1 (stages are used round-robin).
   auto end_tile = [&](int t) {
     wait_vmem_all();
-    __syncthreads();
+    tile_barrier();
     const int dk = ((t + 2) % L::K_STAGES == 0) ? -(L::K_STAGES - 1) * L::TILE_ELEMS : L::TILE_ELEMS;
     const int dv = ((t + 1) % L::V_STAGES == 0) ? -(L::V_STAGES - 1) * L::TILE_ELEMS : L::TILE_ELEMS;
 #pragma unroll
@@ -551,16 +562,16 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   // Tiles whose loads are whole tiles inside the keys: spread over the first step.
   const int n_spread = min(n_tiles, n_inside) - 2;
   for (; t < n_spread; t++) {
-    step(2 * t, std::integral_constant<int, 0>{}, std::true_type{});
-    step(2 * t + 1, std::integral_constant<int, 1>{}, std::false_type{});
+    step(2 * t, HalfTag<0, true>{}, std::true_type{});
+    step(2 * t + 1, HalfTag<1, true>{}, std::false_type{});
     end_tile(t);
   }
   // The last tiles: whatever is left to load (possibly a ragged tile) is issued at once.
   for (; t < n_tiles; t++) {
     if (t + 2 < n_tiles) issue_k(t + 2);
     if (t + 1 < n_tiles) issue_v(t + 1);
-    step(2 * t, std::integral_constant<int, 0>{}, std::false_type{});
-    step(2 * t + 1, std::integral_constant<int, 1>{}, std::false_type{});
+    step(2 * t, HalfTag<0, false>{}, std::false_type{});
+    step(2 * t + 1, HalfTag<1, false>{}, std::false_type{});
     end_tile(t);
   }
   const float l_tot = sum_over_halves(l_run);
