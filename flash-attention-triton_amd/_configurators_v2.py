@@ -3,8 +3,13 @@
 Mirrors ``KernelsConfigV2`` and ``init_to_zero_v2`` of the reference
 (src/flash_attention_triton/_configurators_v2.py:9-93) so that code written against
 ``flash_attention_v2_custom`` keeps working, without importing Triton.  The fields keep their
-names; what they select here is a row of the gfx950 tile/wave table compiled into
-``libfa2_gfx950.so`` rather than Triton meta-parameters.
+names.  The tile shapes of the gfx950 kernels are compiled into ``libfa2_gfx950.so`` (one table row
+per padded head dimension, chosen by the library from the problem), so of the fields below only
+``max_headdim`` (largest accepted head dimension, padding of the log-sum-exp rows) and the
+``SEQUENCE_PARALLEL`` flag of the backward configurations (which backward mode is requested) have
+an effect; the Triton tile, warp and stage counts are accepted and ignored.  The reference's
+kernel-cache key helpers (_configurators_v2.py:40-78) have no counterpart: there is no run-time
+compilation and therefore no kernel cache to key.
 """
 
 from __future__ import annotations
@@ -64,30 +69,6 @@ class KernelsConfigV2:
     max_warps: int
     num_stages: int
     backward_autotune_configs: list = field(default_factory=list)
-
-    def _create_kernel_key(self) -> tuple[tuple[int, int], tuple]:
-        """Immutable key: (compute capability of the current device, all field values).
-
-        Same role as the reference's backward-kernel cache key (_configurators_v2.py:40-55).
-        """
-        cc = torch.cuda.get_device_capability()
-
-        def _serialize(name: str) -> object:
-            attr = getattr(self, name)
-            return self._serialize_bwd(attr) if name == "backward_autotune_configs" else attr
-
-        return cc, tuple(_serialize(name) for name in self.__annotations__)
-
-    def _serialize_bwd(self, bwd_configs: list) -> tuple:
-        """Hashable form of the backward configurations (reference: _configurators_v2.py:57-73)."""
-        return tuple(
-            (tuple(c.kwargs.values()), c.num_warps, c.num_stages, self._hook_name(c.pre_hook))
-            for c in bwd_configs
-        )
-
-    @staticmethod
-    def _hook_name(pre_hook: object) -> str | None:
-        return getattr(pre_hook, "__qualname__", None)
 
     @property
     def deterministic(self) -> bool:

@@ -443,7 +443,10 @@ def flash_attention_v2_custom(
 
     Same contract as the reference (flash_attention_2.py:700-790): the dictionary is keyed by
     ``torch.cuda.get_device_capability()`` of the current device ((9, 5) on MI355X); a missing
-    key raises ValueError.
+    key raises ValueError.  Of the configuration, ``max_headdim`` and the ``SEQUENCE_PARALLEL``
+    flag of the backward configurations are honoured; the Triton tile, warp and stage counts are
+    accepted and ignored (the reference hands them to its kernels, flash_attention_2.py:137-141;
+    here the tile shapes are compiled in, one table row per padded head dimension).
 
     Example:
         configs = {(9, 5): KernelsConfigV2(

@@ -150,9 +150,6 @@ def test_kernels_config_is_a_frozen_record_with_reference_fields(fa):
     with pytest.raises(dataclasses.FrozenInstanceError):
         cfg.block_rows_size = 64
     assert cfg.deterministic is True
-    serial = cfg._serialize_bwd(cfg.backward_autotune_configs)
-    assert serial == (((64, 128, False), 4, 2, "init_to_zero_v2.<locals>.<lambda>"),)
-    hash(serial)
     par = dataclasses.replace(cfg, backward_autotune_configs=[
         fa.BackwardConfig({"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": True})])
     assert par.deterministic is False
