@@ -49,6 +49,16 @@ const fa2_config_info kTable[] = {
 };
 constexpr int kTableRows = sizeof(kTable) / sizeof(kTable[0]);
 
+// Heads dispatched together.  Up to twice the table's group size all heads form one group, so that
+// the whole grid is walked heaviest tile first: with 96 heads, a group of 64 followed by one of 32
+// starts the second group's heaviest tiles halfway through the kernel and they finish alone.
+// Beyond that the table's size applies (a multiple of 8: heads stay on one XCD).
+int head_group(int cfg, int64_t heads) {
+  const int g = kTable[cfg].head_group;
+  if (heads <= 2 * g) return (int)((heads + 7) / 8 * 8);
+  return g;
+}
+
 int pick_config(int headdim) {
   for (int i = 0; i < kTableRows; i++)
     if (headdim <= kTable[i].headdim_padded) return i;
@@ -135,7 +145,7 @@ int fwd_impl(const fa2_fwd_args &a, void *stream) {
   p.headdim = a.headdim;
   p.seqlen_q_rounded = a.seqlen_q_rounded;
   p.n_qtiles = (a.seqlen_q + kFwdBlockQ - 1) / kFwdBlockQ;
-  p.head_group = kTable[cfg].head_group;
+  p.head_group = head_group(cfg, (int64_t)a.batch * a.nheads);
   p.scale = a.softmax_scale;
   p.scale_log2 = a.softmax_scale * fa2::kLog2e;
   p.vec = vec_ok(p.q, a.headdim) && vec_ok(p.k, a.headdim) && vec_ok(p.v, a.headdim) && vec_ok(p.o, a.headdim);
@@ -216,7 +226,7 @@ int bwd_impl(const fa2_bwd_args &a, void *stream) {
   p.seqlen_k = a.seqlen_k;
   p.headdim = a.headdim;
   p.seqlen_q_rounded = a.seqlen_q_rounded;
-  p.head_group = kTable[cfg].head_group;
+  p.head_group = head_group(cfg, (int64_t)a.batch * a.nheads);
   p.scale = a.softmax_scale;
   p.scale_log2 = a.softmax_scale * fa2::kLog2e;
   p.vec = vec_ok(p.q, a.headdim) && vec_ok(p.k, a.headdim) && vec_ok(p.v, a.headdim) &&
@@ -229,6 +239,9 @@ int bwd_impl(const fa2_bwd_args &a, void *stream) {
   const int64_t bh = (int64_t)a.batch * a.nheads;
 
   fa2::BwdParams pk = p, pq = p;
+  // The dK/dV kernel keeps the table's group size at every head count: with one or two workgroups
+  // per CU its drain is short either way, and measured at 96 heads the single group is 1-2 % slower.
+  pk.head_group = kTable[cfg].head_group;
   pk.n_tiles = (a.seqlen_k + kDkvBlockKV - 1) / kDkvBlockKV;
   pq.n_tiles = (a.seqlen_q + kDqBlockQ - 1) / kDqBlockQ;
   const int64_t nwg_k = pk.n_tiles * bh, nwg_q = pq.n_tiles * bh;
