@@ -249,8 +249,10 @@ class FlashAttentionV2Function(torch.autograd.Function):
         initial_dtype = q.dtype
         compute_dtype = _compute_dtype(initial_dtype)
 
-        # No-ops for contiguous fp16/bf16 inputs.
-        q, k, v = [proj.contiguous().to(compute_dtype) for proj in (q, k, v)]
+        # Contiguous fp16/bf16 inputs are used as they are.
+        if not (q.dtype == k.dtype == v.dtype == compute_dtype
+                and q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+            q, k, v = [proj.contiguous().to(compute_dtype) for proj in (q, k, v)]
 
         output, lse, ctx.softmax_scale = _flash_attention_forward(
             q,
@@ -270,7 +272,8 @@ class FlashAttentionV2Function(torch.autograd.Function):
         ctx.save_for_backward(q, k, v, output, lse)
         ctx.kernels_config = kernels_config
 
-        return output.contiguous().to(initial_dtype)
+        # `output` is contiguous (allocated like the contiguous q).
+        return output if initial_dtype == compute_dtype else output.to(initial_dtype)
 
     @staticmethod
     def backward(ctx, d_output):  # noqa: ANN001, ANN205
