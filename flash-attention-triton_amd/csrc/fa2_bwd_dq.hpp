@@ -381,6 +381,13 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   const int qrow = q0w + c;
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
+  // Where sixteen registers are to spare, the dP chain of every block starts from -delta instead of
+  // zero (the MFMA's C operand), so that dS = P * dP needs no subtraction.  At 128 columns the
+  // kernel already fills the 256 registers that two workgroups per CU leave a wave.
+  constexpr bool DELTA_IN_CHAIN = DP <= 96;
+  const f32x16 dp_start = DELTA_IN_CHAIN ? splat16(-delta) : zero;
+  const float delta_sub = DELTA_IN_CHAIN ? 0.f : delta;
+
   wait_vmem_all();
   __syncthreads();
 
@@ -410,7 +417,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
     const unsigned kdst = lds_base + 2u * (unsigned)(L::K_BASE + (kt % L::K_STAGES) * L::TILE_ELEMS);
     const unsigned vdst = lds_base + 2u * (unsigned)(L::V_BASE + (vt % L::V_STAGES) * L::TILE_ELEMS);
     constexpr int HOFF = HALF * BLK * LP;
-    f32x16 s = zero, dp = zero;
+    f32x16 s = zero, dp;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       s = Elem<T>::mfma(ring[ks], qf[ks], s);
@@ -421,7 +428,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
     const bool need_mask = j >= n_full;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      dp = Elem<T>::mfma(ring[ks], gf[ks], dp);
+      dp = Elem<T>::mfma(ring[ks], gf[ks], ks == 0 ? dp_start : dp);
       if (SPREAD && ks % LOAD_EVERY == 0 && ks / LOAD_EVERY < LOADS) kload.issue_one(kt * BKV, kdst, ks / LOAD_EVERY);
       {
         s16x4 a0 = lds_read_tr(klo[ks % DB] + HOFF + 16 * (ks / DB) * LP);
@@ -443,7 +450,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
     // dS of the first 16 keys before the dQ MFMAs that need them, the rest beside those MFMAs.
     f32x8 lo, hi;
 #pragma unroll
-    for (int i = 0; i < 8; i++) lo[i] = s[i] * (dp[i] - delta);
+    for (int i = 0; i < 8; i++) lo[i] = DELTA_IN_CHAIN ? s[i] * dp[i] : s[i] * (dp[i] - delta_sub);
     s16x8 dsf[2];
     dsf[0] = Elem<T>::pack8(lo);
 #pragma unroll
@@ -455,7 +462,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
       if (slot < HALF_SLOTS) {
 #pragma unroll
         for (int i = part(8, HALF_SLOTS, slot); i < part(8, HALF_SLOTS, slot + 1); i++)
-          hi[i] = s[8 + i] * (dp[8 + i] - delta);
+          hi[i] = DELTA_IN_CHAIN ? s[8 + i] * dp[8 + i] : s[8 + i] * (dp[8 + i] - delta_sub);
         asm volatile("" : "+v"(hi));
         if (slot == HALF_SLOTS - 1) dsf[1] = Elem<T>::pack8(hi);
       }

@@ -141,6 +141,17 @@ __device__ __forceinline__ float sum_over_halves(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Sixteen copies of one value, kept in sixteen registers: the form an MFMA takes as its C operand.
+// The empty asm statement hides from the optimiser that the registers are equal; otherwise it
+// rebuilds the block with sixteen moves in front of every use.
+__device__ __forceinline__ f32x16 splat16(float x) {
+  f32x16 r;
+#pragma unroll
+  for (int i = 0; i < 16; i++) r[i] = x;
+  asm volatile("" : "+v"(r));
+  return r;
+}
+
 // Load 8 consecutive 16-bit elements row[d0 .. d0+7], zero beyond `headdim` or when the row is
 // out of range.  `vec` (uniform) says 16-byte loads are legal: headdim % 8 == 0 and every row
 // start is 16-byte aligned.
