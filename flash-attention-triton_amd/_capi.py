@@ -15,12 +15,13 @@ import threading
 # The in-tree build; FA2_GFX950_LIBRARY names another build of the same ABI (e.g. one under test).
 LIBRARY_PATH = pathlib.Path(os.environ.get("FA2_GFX950_LIBRARY") or
                             pathlib.Path(__file__).resolve().parent / "csrc" / "libfa2_gfx950.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 FA2_DTYPE_F16 = 0
 FA2_DTYPE_BF16 = 1
 FA2_CONFIG_AUTO = -1
 FA2_MAX_HEADDIM = 256
+FA2_NOALLOC_MAX_ROWS = 4 << 20
 
 _i, _i64, _f, _p = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -78,6 +79,7 @@ SIGNATURES = {
     "fa2_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 7),
     "fa2_bwd": (_i, [_p] * 10 + [_i] * 6 + [_i64] * 21 + [_f, _i, _i, _i, _p]),
     "fa2_bwd_fused": (_i, [_p] * 11 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p]),
+    "fa2_bwd_fused_noalloc": (_i, [_p] * 9 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p]),
     "fa2_fwd_packed": (_i, [ctypes.POINTER(FwdArgs), _p]),
     "fa2_bwd_packed": (_i, [ctypes.POINTER(BwdArgs), _p]),
 }

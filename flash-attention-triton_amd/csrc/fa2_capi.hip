@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -274,6 +275,37 @@ int bwd_impl(const fa2_bwd_args &a, void *stream) {
 
 fa2_tensor make_tensor(const void *ptr, int64_t sb, int64_t sh, int64_t ss) { return fa2_tensor{ptr, sb, sh, ss}; }
 
+// ---- delta scratch of fa2_bwd_fused_noalloc ---------------------------------------------------
+// fa2_bwd_fused needs batch * nheads * seqlen_q_rounded floats of scratch (delta) from its caller.
+// The variant for callers that cannot allocate keeps that scratch here, in a device array that
+// every GPU the library runs on holds until the process ends.  In host code `scratch` is only a
+// handle for hipGetSymbolAddress: the device address differs per GPU and is looked up once per
+// device (with that device current) and kept in g_scratch_addr.
+constexpr size_t kScratchFloats = FA2_NOALLOC_MAX_ROWS;
+static __device__ __align__(256) float scratch[kScratchFloats];
+constexpr int kMaxDevices = 64;
+std::atomic<float *> g_scratch_addr[kMaxDevices];
+
+int scratch_on_current_device(float **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(FA2_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(FA2_ERR_TOO_LARGE, "device ordinal %d outside [0, %d)", dev, kMaxDevices);
+  float *addr = g_scratch_addr[dev].load(std::memory_order_acquire);
+  if (addr == nullptr) {
+    // Two threads may both get here the first time; they find the same address.
+    void *sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || sym == nullptr)
+      return fail(FA2_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    addr = static_cast<float *>(sym);
+    g_scratch_addr[dev].store(addr, std::memory_order_release);
+  }
+  *out = addr;
+  return FA2_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -436,6 +468,35 @@ int fa2_bwd_fused(const void *q, const void *k, const void *v, const void *o, co
   a.deterministic = deterministic;
   a.config_id = config_id;
   return bwd_impl(a, stream);
+}
+
+int fa2_bwd_fused_noalloc(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                          const float *lse, void *dq, void *dk, void *dv, int batch, int nheads,
+                          int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded, int64_t q_sb,
+                          int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                          int64_t v_sb, int64_t v_sh, int64_t v_ss, int64_t o_sb, int64_t o_sh,
+                          int64_t o_ss, int64_t do_sb, int64_t do_sh, int64_t do_ss, int64_t dq_sb,
+                          int64_t dq_sh, int64_t dq_ss, int64_t dk_sb, int64_t dk_sh, int64_t dk_ss,
+                          int64_t dv_sb, int64_t dv_sh, int64_t dv_ss, float softmax_scale, int dtype,
+                          int deterministic, int config_id, void *stream) {
+  if (o == nullptr) return fail(FA2_ERR_NULL_POINTER, "o is NULL");
+  if (batch <= 0 || nheads <= 0 || seqlen_q_rounded <= 0)
+    return fail(FA2_ERR_BAD_SHAPE, "sizes must be positive: batch=%d nheads=%d seqlen_q_rounded=%d", batch,
+                nheads, seqlen_q_rounded);
+  const uint64_t rows = (uint64_t)batch * (uint64_t)nheads * (uint64_t)seqlen_q_rounded;
+  if (rows > kScratchFloats)
+    return fail(FA2_ERR_TOO_LARGE,
+                "batch*nheads*seqlen_q_rounded = %llu rows exceed the %llu rows of built-in scratch "
+                "(FA2_NOALLOC_MAX_ROWS); use fa2_bwd_fused with a caller-supplied delta buffer",
+                (unsigned long long)rows, (unsigned long long)kScratchFloats);
+  float *delta = nullptr;
+  if (int rc = scratch_on_current_device(&delta)) return rc;
+  // Every row of delta the kernels read is written earlier in the same call (by the dQ kernel or
+  // the preprocess kernel), so nothing left over from an earlier call has to be cleared.
+  return fa2_bwd_fused(q, k, v, o, d_o, lse, delta, nullptr, dq, dk, dv, batch, nheads, seqlen_q, seqlen_k,
+                       headdim, seqlen_q_rounded, q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb,
+                       o_sh, o_ss, do_sb, do_sh, do_ss, dq_sb, dq_sh, dq_ss, dk_sb, dk_sh, dk_ss, dv_sb,
+                       dv_sh, dv_ss, softmax_scale, dtype, deterministic, config_id, stream);
 }
 
 }  // extern "C"

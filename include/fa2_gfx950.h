@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define FA2_ABI_VERSION 2
+#define FA2_ABI_VERSION 3
 
 /* Largest head dimension the kernels accept (the table's `max_headdim`). */
 #define FA2_MAX_HEADDIM 256
@@ -55,6 +55,9 @@ typedef enum fa2_dtype {
   FA2_DTYPE_F16 = 0, /* IEEE half: the reference's only compute type (flash_attention_2.py:90) */
   FA2_DTYPE_BF16 = 1 /* bfloat16 on bf16 MFMA; the reference down-casts bf16 to fp16 instead */
 } fa2_dtype;
+
+/* Rows (batch * nheads * seqlen_q_rounded) fa2_bwd_fused_noalloc has built-in scratch for: 16 MiB. */
+#define FA2_NOALLOC_MAX_ROWS (4u << 20)
 
 /* Ask the table to choose (pass as config_id). */
 #define FA2_CONFIG_AUTO (-1)
@@ -237,6 +240,33 @@ int fa2_bwd_fused(const void *q, const void *k, const void *v, const void *o, co
                   int64_t dk_stride_batch, int64_t dk_stride_head, int64_t dk_stride_seq,
                   int64_t dv_stride_batch, int64_t dv_stride_head, int64_t dv_stride_seq,
                   float softmax_scale, int dtype, int deterministic, int config_id, void *stream);
+
+/*
+ * fa2_bwd_fused for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc): same arguments without `delta` and
+ * `workspace`, same dq, dk, dv bit for bit.  It has no counterpart in the reference, whose launcher
+ * allocates delta itself (flash_attention_2.py:195).  The delta scratch lives in a device array
+ * inside the library, FA2_NOALLOC_MAX_ROWS floats (16 MiB) on every GPU the library runs on, held
+ * until the process ends; the call allocates and frees nothing and never synchronises.
+ * batch * nheads * seqlen_q_rounded above FA2_NOALLOC_MAX_ROWS is refused with
+ * FA2_ERR_TOO_LARGE.  All calls on one GPU share that array: two calls that may overlap there
+ * (different streams, different threads) race on it - keep them on one stream or use
+ * fa2_bwd_fused with separate buffers.  Nothing left in the array by an earlier call is read: each
+ * call writes every row of delta before it reads it.  The first call on a device looks up the
+ * array's address (hipGetSymbolAddress); make that call outside stream capture.
+ */
+int fa2_bwd_fused_noalloc(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                          const float *lse, void *dq, void *dk, void *dv,
+                          int batch, int nheads, int seqlen_q, int seqlen_k, int headdim, int seqlen_q_rounded,
+                          int64_t q_stride_batch, int64_t q_stride_head, int64_t q_stride_seq,
+                          int64_t k_stride_batch, int64_t k_stride_head, int64_t k_stride_seq,
+                          int64_t v_stride_batch, int64_t v_stride_head, int64_t v_stride_seq,
+                          int64_t o_stride_batch, int64_t o_stride_head, int64_t o_stride_seq,
+                          int64_t do_stride_batch, int64_t do_stride_head, int64_t do_stride_seq,
+                          int64_t dq_stride_batch, int64_t dq_stride_head, int64_t dq_stride_seq,
+                          int64_t dk_stride_batch, int64_t dk_stride_head, int64_t dk_stride_seq,
+                          int64_t dv_stride_batch, int64_t dv_stride_head, int64_t dv_stride_seq,
+                          float softmax_scale, int dtype, int deterministic, int config_id, void *stream);
 
 /*
  * The backward with its arguments in one record: fa2_bwd when args->o.ptr is NULL, fa2_bwd_fused
