@@ -415,7 +415,11 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       dkacc[db][i] = 0.f;
       dvacc[db][i] = 0.f;
     }
+  // Element i of a block that starts at query row qb is row qb + 4h + 8 (i / 4) + i % 4; it is kept
+  // when key column <= row < seqlen_q, tested as one unsigned compare: (row - column) < (seqlen_q - column).
   const int kvcol = kv0w + c;
+  const int row_shift = 4 * h - kvcol;  // row - column = qb + 8 (i / 4) + i % 4 + row_shift
+  const unsigned row_span = (unsigned)max(seqlen_q - kvcol, 0);
 
 #pragma unroll
   for (int t = 0; t < L::STAGES; t++) {
@@ -482,6 +486,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     }
     // ---- dP = dO V^T (ringb: dO rows -> Q^T); exponentials under the MFMAs -------------------
     f32x16 pr;
+    const int rel = qb + row_shift;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       // The chain starts from -delta, so that dS = P * dP needs no subtraction.
@@ -500,10 +505,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 #pragma unroll
       for (int i = part(16, KS, ks); i < part(16, KS, ks + 1); i++) {
         float x = fast_exp2(s[i] * scale_log2 - l4[i >> 2][i & 3]);
-        if (MASKED) {
-          const int qr = qb + 8 * (i >> 2) + 4 * h + (i & 3);
-          if (kvcol > qr || qr >= seqlen_q) x = 0.f;
-        }
+        if (MASKED && (unsigned)(rel + (8 * (i >> 2) + (i & 3))) >= row_span) x = 0.f;
         pr[i] = x;
       }
       asm volatile("" : "+v"(pr));

@@ -378,7 +378,10 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   for (int db = 0; db < DB; db++)
 #pragma unroll
     for (int i = 0; i < 16; i++) dqacc[db][i] = 0.f;
-  const int qrow = q0w + c;
+  // Element i of a score block that starts at key kv0 is key kv0 + 4h + 8 (i / 4) + i % 4; it is kept
+  // when that key is at most min(query row, last key): one subtraction per block and one compare
+  // with a constant per element.
+  const int key_limit = min(q0w + c, seqlen_k - 1) - 4 * h;
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // Where sixteen registers are to spare, the dP chain of every block starts from -delta instead of
@@ -425,7 +428,16 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
       ring[ks] = lds_read_128(vrow[ks] + HOFF);
       __builtin_amdgcn_sched_barrier(0);
     }
-    const bool need_mask = j >= n_full;
+    if (j >= n_full) {
+      // Diagonal and ragged blocks: masked scores become -inf, their probabilities 0.  The empty asm
+      // statement keeps this a branch that interior blocks skip (the test is cheap enough that the
+      // optimiser would otherwise run it for every block).
+      asm volatile("");
+      const int lim = key_limit - j * BLK;
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        if (8 * (i >> 2) + (i & 3) > lim) s[i] = -INFINITY;
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       dp = Elem<T>::mfma(ring[ks], gf[ks], ks == 0 ? dp_start : dp);
@@ -437,12 +449,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
       }
 #pragma unroll
       for (int i = part(16, KS, ks); i < part(16, KS, ks + 1); i++) {
-        float pr = fast_exp2(s[i] * scale_log2 - lse2);
-        if (need_mask) {
-          const int kv = j * BLK + 8 * (i >> 2) + 4 * h + (i & 3);
-          if (kv > qrow || kv >= seqlen_k) pr = 0.f;
-        }
-        s[i] = pr;
+        s[i] = fast_exp2(s[i] * scale_log2 - lse2);
       }
       asm volatile("" : "+v"(s));
       __builtin_amdgcn_sched_barrier(0);
