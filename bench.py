@@ -333,6 +333,20 @@ def main() -> int:
         torch.cuda.synchronize()
         step_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # The same steps with PyTorch's backward engine kept on the calling thread.  By default the
+    # engine hands the backward of CUDA tensors to a worker thread and waits for it; at the smallest
+    # workloads that hand-off (tens of microseconds of host time) is longer than the kernels.
+    # Reported beside ms_per_step, never instead of it.
+    with torch.autograd.set_multithreading_enabled(False):
+        for _ in range(max(args.warmup, 1)):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        step_ms_one_thread = (time.perf_counter() - t0) * 1e3 / args.steps
+
     settle(fwd_only)
     for _ in range(max(args.warmup, 1)):
         fwd_only()
@@ -397,6 +411,7 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": step_ms,
+        "ms_per_step_autograd_on_calling_thread": step_ms_one_thread,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -384,12 +384,9 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   const int key_limit = min(q0w + c, seqlen_k - 1) - 4 * h;
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  // Where sixteen registers are to spare, the dP chain of every block starts from -delta instead of
-  // zero (the MFMA's C operand), so that dS = P * dP needs no subtraction.  At 128 columns the
-  // kernel already fills the 256 registers that two workgroups per CU leave a wave.
-  constexpr bool DELTA_IN_CHAIN = DP <= 96;
-  const f32x16 dp_start = DELTA_IN_CHAIN ? splat16(-delta) : zero;
-  const float delta_sub = DELTA_IN_CHAIN ? 0.f : delta;
+  // The dP chain of every block starts from -delta instead of zero (the MFMA's C operand), so that
+  // dS = P * dP needs no subtraction.  Costs sixteen registers (255 of 256 in use at 128 columns).
+  const f32x16 dp_start = splat16(-delta);
 
   wait_vmem_all();
   __syncthreads();
@@ -457,7 +454,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
     // dS of the first 16 keys before the dQ MFMAs that need them, the rest beside those MFMAs.
     f32x8 lo, hi;
 #pragma unroll
-    for (int i = 0; i < 8; i++) lo[i] = DELTA_IN_CHAIN ? s[i] * dp[i] : s[i] * (dp[i] - delta_sub);
+    for (int i = 0; i < 8; i++) lo[i] = s[i] * dp[i];
     s16x8 dsf[2];
     dsf[0] = Elem<T>::pack8(lo);
 #pragma unroll
@@ -469,7 +466,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
       if (slot < HALF_SLOTS) {
 #pragma unroll
         for (int i = part(8, HALF_SLOTS, slot); i < part(8, HALF_SLOTS, slot + 1); i++)
-          hi[i] = DELTA_IN_CHAIN ? s[8 + i] * dp[8 + i] : s[8 + i] * (dp[8 + i] - delta_sub);
+          hi[i] = s[8 + i] * dp[8 + i];
         asm volatile("" : "+v"(hi));
         if (slot == HALF_SLOTS - 1) dsf[1] = Elem<T>::pack8(hi);
       }
