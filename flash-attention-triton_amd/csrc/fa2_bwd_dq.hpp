@@ -403,11 +403,14 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   //     C: dQ^T += K^T dS^T       ring <- next block's K rows second half of the dS arithmetic
   constexpr int LOADS = TileLoader<DP, BKV, kDqWaves>::LOADS;
   constexpr int LOAD_EVERY = KS / LOADS;
-  auto block = [&](int j, auto half_tag, auto spread_tag) __attribute__((always_inline)) {
+  // INNER blocks lie in tiles that end before the workgroup's first query row: they are every
+  // wave's own and need no mask, so the two tests fold away.
+  auto block = [&](int j, auto half_tag, auto spread_tag, auto inner_tag) __attribute__((always_inline)) {
     constexpr int HALF = decltype(half_tag)::value;
     constexpr bool SPREAD = decltype(spread_tag)::value;
+    constexpr bool INNER = decltype(inner_tag)::value;
     const int kt = j / 2 + 2, vt = j / 2 + 1;  // tiles loaded during this block (SPREAD)
-    if (j >= n_mine) {
+    if (!INNER && j >= n_mine) {
       if (SPREAD) {  // not reached: skipped blocks lie in the last two tiles, which load nothing
         issue_k(kt);
         issue_v(vt);
@@ -425,7 +428,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
       ring[ks] = lds_read_128(vrow[ks] + HOFF);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (j >= n_full) {
+    if (!INNER && j >= n_full) {
       // Diagonal and ragged blocks: masked scores become -inf, their probabilities 0.  The empty asm
       // statement keeps this a branch that interior blocks skip (the test is cheap enough that the
       // optimiser would otherwise run it for every block).
@@ -491,12 +494,12 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
     }
   };
   auto tile = [&](int t, auto spread_tag) __attribute__((always_inline)) {
-    block(2 * t, std::integral_constant<int, 0>{}, spread_tag);
+    block(2 * t, std::integral_constant<int, 0>{}, spread_tag, spread_tag);
     // knext -> K tile t+1 before the second block prefetches from it.
     const int dk = k_step(t);
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) knext[ks] += dk;
-    block(2 * t + 1, std::integral_constant<int, 1>{}, std::false_type{});
+    block(2 * t + 1, std::integral_constant<int, 1>{}, std::false_type{}, spread_tag);
     end_tile(t);
   };
   int t = 0;

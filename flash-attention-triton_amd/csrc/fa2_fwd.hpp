@@ -493,7 +493,9 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
       if (ks == KS - 1) asm volatile("" : "+v"(w[1]));
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (j + 1 >= n_full) apply_mask(sc, (j + 1) * BLK);
+    // S_{j+1} of a SPREAD step is the second half of a tile that ends before the workgroup's first
+    // query row: never masked.  (The step after it may produce the first block of the diagonal.)
+    if (!SPREAD && j + 1 >= n_full) apply_mask(sc, (j + 1) * BLK);
     const s16x8 pf[2] = {__builtin_bit_cast(s16x8, w[0]), __builtin_bit_cast(s16x8, w[1])};
     const float mc = m_ref * scale_log2;
     float lsum[2] = {0.f, 0.f};  // this lane's sum of the new probabilities, in two chains
