@@ -355,12 +355,10 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       sl[BQ + tid] = -delta_reg;  // negated: it is the accumulator the dP MFMAs start from
     }
   };
-  // Prologue: every global load of the first three tiles and of this wave's K and V rows is
-  // issued before anything waits, so that the workgroup pays one memory latency, not one per
-  // tile.
-#pragma unroll
-  for (int t = 0; t < L::STAGES; t++)
-    if (t < n_tiles) issue_tile(t);
+  // Prologue: the first tile and this wave's K and V rows are requested before anything waits;
+  // tiles 1 and 2 follow right after the first barrier and land while tile 0 is being multiplied,
+  // so the first MFMA waits for one tile, not three.
+  if (0 < n_tiles) issue_tile(0);
 
   // B operands: lane (c, h) holds row kv0w + c of K and of V, columns 16 ks + 8 h + j.
   s16x8 kf[KS], vf[KS];
@@ -429,6 +427,9 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   }
   wait_vmem_all();
   __syncthreads();
+#pragma unroll
+  for (int t = 1; t < L::STAGES; t++)
+    if (t < n_tiles) issue_tile(t);
   // Two rings of A fragments, preloaded with the Q rows and the dO rows of block 0.
   s16x8 ring[KS], ringb[KS];
 #pragma unroll
