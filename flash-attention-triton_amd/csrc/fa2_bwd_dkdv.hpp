@@ -280,7 +280,9 @@ struct DkvDirectLayout {
       (STAGES * STAGE_ELEMS > PATCH_ELEMS) ? STAGES * STAGE_ELEMS : PATCH_ELEMS;
 };
 
-template <typename T, int DP, int BQ>
+// PAD: the head dimension is a multiple of 8 below DP; the columns beyond it are zeros in LDS and in
+// the register fragments, and are not stored.
+template <typename T, int DP, int BQ, bool PAD>
 __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_direct_kernel(const BwdParams p) {
   using L = DkvDirectLayout<DP, BQ>;
   constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
@@ -314,7 +316,8 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   const float *LSE = p.lse + (int64_t)bh * p.seqlen_q_rounded;
   const float *DELTA = p.delta + (int64_t)bh * p.seqlen_q_rounded;
 
-  const TileLoader<DP, BQ, kDkvWaves> qload(Q, p.q.stride_seq), gload(DO, p.d_o.stride_seq);
+  const int hdim = PAD ? p.headdim : DP;
+  const TileLoader<DP, BQ, kDkvWaves, PAD> qload(Q, p.q.stride_seq, hdim / 8), gload(DO, p.d_o.stride_seq, hdim / 8);
   const int seqlen_q = p.seqlen_q;
   const float scale_log2 = p.scale_log2;
 
@@ -326,6 +329,10 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   const int n_diag = min(n_tiles, (kv0 + kDkvBlockKV - q_begin + BQ - 1) / BQ);
 
   const unsigned lds_base = lds_u32(smem);  // LDS byte address of smem
+  if (PAD) {
+    zero_lds<NTHREADS>(smem, L::STAGES * L::STAGE_ELEMS);
+    __syncthreads();
+  }
   auto issue_tile = [&](int t) {
     const unsigned dst = lds_base + 2u * (unsigned)((t % L::STAGES) * L::STAGE_ELEMS);
     const int row0 = q_begin + t * BQ;
@@ -369,8 +376,8 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     const short *vp = V + (int64_t)row * p.v.stride_seq;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      kf[ks] = load_chunk(kp, 16 * ks + 8 * h, DP, ok, true);
-      vf[ks] = load_chunk(vp, 16 * ks + 8 * h, DP, ok, true);
+      kf[ks] = load_chunk(kp, 16 * ks + 8 * h, hdim, ok, true);
+      vf[ks] = load_chunk(vp, 16 * ks + 8 * h, hdim, ok, true);
     }
   }
   // Statistics of the first three tiles: loaded now, written to LDS just before the first
@@ -445,7 +452,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     constexpr int HALF = decltype(half_tag)::value;
     constexpr bool MASKED = decltype(masked_tag)::value;
     constexpr bool SPREAD = decltype(spread_tag)::value;
-    constexpr int LOADS = TileLoader<DP, BQ, kDkvWaves>::LOADS;
+    constexpr int LOADS = TileLoader<DP, BQ, kDkvWaves, PAD>::LOADS;
     constexpr int EVERY = 4 * KS / (2 * LOADS);  // units between loads: both tiles' loads fit the block
     static_assert(EVERY >= 1 && (2 * LOADS - 1) * EVERY < 4 * KS, "the block must have room for both tiles' loads");
     const unsigned ldst = lds_base + 2u * (unsigned)((lt % L::STAGES) * L::STAGE_ELEMS);
@@ -579,12 +586,12 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
 
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(dvacc, 1.0f, patch, DV + (int64_t)kv0w * p.dv.stride_seq,
-                              p.dv.stride_seq, p.seqlen_k - kv0w, DP, true);
+                              p.dv.stride_seq, p.seqlen_k - kv0w, hdim, true);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   store_transposed_acc<T, DP>(dkacc, p.scale, patch, DK + (int64_t)kv0w * p.dk.stride_seq,
-                              p.dk.stride_seq, p.seqlen_k - kv0w, DP, true);
+                              p.dk.stride_seq, p.seqlen_k - kv0w, hdim, true);
 }
 
 }  // namespace fa2

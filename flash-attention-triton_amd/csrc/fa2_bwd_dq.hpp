@@ -266,7 +266,9 @@ struct DqDirectLayout {
 // With FUSE_DELTA the kernel also computes delta = rowsum(O * dO) for its query rows (it holds
 // the dO rows anyway), uses it and writes it out for the dK/dV kernel, which then has to be
 // launched after this one; the separate preprocess launch disappears.
-template <typename T, int DP, int BKV, bool FUSE_DELTA>
+// PAD: the head dimension is a multiple of 8 below DP; the columns beyond it are zeros in LDS and in
+// the register fragments, and are not stored.
+template <typename T, int DP, int BKV, bool FUSE_DELTA, bool PAD>
 __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const BwdParams p) {
   using L = DqDirectLayout<DP, BKV>;
   constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
@@ -295,7 +297,8 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   const short *DO = (const short *)p.d_o.ptr + b * p.d_o.stride_batch + hd * p.d_o.stride_head;
   short *DQ = (short *)p.dq.ptr + b * p.dq.stride_batch + hd * p.dq.stride_head;
 
-  const TileLoader<DP, BKV, kDqWaves> kload(K, p.k.stride_seq), vload(V, p.v.stride_seq);
+  const int hdim = PAD ? p.headdim : DP;
+  const TileLoader<DP, BKV, kDqWaves, PAD> kload(K, p.k.stride_seq, hdim / 8), vload(V, p.v.stride_seq, hdim / 8);
   const int seqlen_k = p.seqlen_k;
   const float scale_log2 = p.scale_log2;
 
@@ -306,6 +309,10 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   const int n_inside = seqlen_k / BKV;
 
   const unsigned lds_base = lds_u32(smem);  // LDS byte address of smem
+  if (PAD) {
+    zero_lds<64 * kDqWaves>(smem, L::STAGE_ELEMS);
+    __syncthreads();
+  }
   auto issue_k = [&](int t) {
     const unsigned dst = lds_base + 2u * (unsigned)(L::K_BASE + (t % L::K_STAGES) * L::TILE_ELEMS);
     if (t < n_inside) kload.issue(t * BKV, dst); else kload.issue_clamped(t * BKV, seqlen_k, dst);
@@ -329,8 +336,8 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
     const short *gp = DO + (int64_t)row * p.d_o.stride_seq;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      qf[ks] = load_chunk(qp, 16 * ks + 8 * h, DP, ok, true);
-      gf[ks] = load_chunk(gp, 16 * ks + 8 * h, DP, ok, true);
+      qf[ks] = load_chunk(qp, 16 * ks + 8 * h, hdim, ok, true);
+      gf[ks] = load_chunk(gp, 16 * ks + 8 * h, hdim, ok, true);
     }
     if (ok) lse2 = p.lse[(int64_t)bh * p.seqlen_q_rounded + row] * kLog2e;
     if (FUSE_DELTA) {
@@ -339,7 +346,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
       float part = 0.f;  // this lane's half of the row: columns 16 ks + 8 h + j
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
-        const s16x8 of = load_chunk(op, 16 * ks + 8 * h, DP, ok, true);
+        const s16x8 of = load_chunk(op, 16 * ks + 8 * h, hdim, ok, true);
 #pragma unroll
         for (int j = 0; j < 8; j++) part += Elem<T>::to_float(of[j]) * Elem<T>::to_float(gf[ks][j]);
       }
@@ -401,7 +408,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
   //     A: S^T = K Q^T            ring <- V rows              (loads of V tile t+1 when SPREAD)
   //     B: dP^T = V dO^T          ring <- K^T fragments       exponentials of S; loads of K tile t+2
   //     C: dQ^T += K^T dS^T       ring <- next block's K rows second half of the dS arithmetic
-  constexpr int LOADS = TileLoader<DP, BKV, kDqWaves>::LOADS;
+  constexpr int LOADS = TileLoader<DP, BKV, kDqWaves, PAD>::LOADS;
   constexpr int LOAD_EVERY = KS / LOADS;
   // INNER blocks lie in tiles that end before the workgroup's first query row: they are every
   // wave's own and need no mask, so the two tests fold away.
@@ -513,7 +520,7 @@ __global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const B
 
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(dqacc, p.scale, patch, DQ + (int64_t)q0w * p.dq.stride_seq,
-                              p.dq.stride_seq, p.seqlen_q - q0w, DP, true);
+                              p.dq.stride_seq, p.seqlen_q - q0w, hdim, true);
 }
 
 

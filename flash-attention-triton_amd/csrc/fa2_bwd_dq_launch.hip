@@ -5,14 +5,22 @@
 namespace fa2 {
 namespace {
 
+template <typename T, bool FUSE_DELTA, bool PAD>
+void launch_direct_pad(int dp, const BwdParams &p, dim3 grid, dim3 block, hipStream_t s) {
+  switch (dp) {
+    case 32: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 32, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
+    case 64: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 64, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
+    case 96: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 96, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 128, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
+  }
+}
+
 template <typename T, bool FUSE_DELTA>
 void launch_direct(int dp, const BwdParams &p, dim3 grid, dim3 block, hipStream_t s) {
-  switch (dp) {
-    case 32: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 32, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
-    case 64: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 64, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
-    case 96: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 96, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 128, kDqBlockKV, FUSE_DELTA>), grid, block, 0, s, p); break;
-  }
+  if (p.headdim == dp)
+    launch_direct_pad<T, FUSE_DELTA, false>(dp, p, grid, block, s);
+  else
+    launch_direct_pad<T, FUSE_DELTA, true>(dp, p, grid, block, s);
 }
 
 template <typename T>

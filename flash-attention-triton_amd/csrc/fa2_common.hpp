@@ -325,11 +325,21 @@ constexpr int part(int n, int units, int u) { return n * u / units; }
 // complete after it.
 __device__ __forceinline__ void tile_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
+// Zero `elems` halves of LDS (a multiple of 8 per thread step) with the whole workgroup.  The
+// padded kernels do this once before their first tile load: tile loads never touch the slots of
+// columns beyond the head dimension, which the MFMAs read as part of their DP-wide fragments.
+template <int NTHREADS>
+__device__ __forceinline__ void zero_lds(short *smem, int elems) {
+  const fa2::s16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int i = threadIdx.x * 8; i < elems; i += NTHREADS * 8) *reinterpret_cast<fa2::s16x8 *>(smem + i) = z;
+}
+
 // Streams ROWS x DP tiles of a (seqlen, headdim) matrix into swizzled LDS (row pitch lds_pitch(DP))
 // with LDS-direct loads.  All NW waves of the workgroup take part; each wave issues LOADS loads of
 // 1 KiB of LDS per tile.  A lane owns one 16-byte slot of a row; lanes whose slot holds no data
-// (DP < pitch) are switched off for the load.
-template <int DP, int ROWS, int NW>
+// (DP < pitch, or with PAD a head dimension of `chunks` 16-byte chunks below DP) are switched off
+// for the load.
+template <int DP, int ROWS, int NW, bool PAD = false>
 struct TileLoader {
   static constexpr int LP = lds_pitch(DP);
   static constexpr int CPR = LP / 8;    // chunk slots per row
@@ -350,12 +360,15 @@ struct TileLoader {
   unsigned voff;      // byte offset of this lane inside a tile for load 0
   bool active;        // this lane's slot holds data
 
-  __device__ __forceinline__ TileLoader(const short *base_, int64_t stride_) : base(base_), stride(stride_) {
+  static constexpr bool ALL_ACTIVE = LP == DP && !PAD;  // every slot of a row holds data
+
+  __device__ __forceinline__ TileLoader(const short *base_, int64_t stride_, int chunks = DP / 8)
+      : base(base_), stride(stride_) {
     const int lane = threadIdx.x & 63;
     wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     row_in = wave * RPL + lane / CPR;
     chunk = (lane % CPR) ^ swz<LP>(row_in);
-    active = LP == DP || chunk < DP / 8;
+    active = ALL_ACTIVE || chunk < (PAD ? chunks : DP / 8);
     voff = 2u * (unsigned)(row_in * (int)stride + chunk * 8);
   }
 
@@ -369,7 +382,7 @@ struct TileLoader {
   // between other work.
   __device__ __forceinline__ void issue_one(int row0, unsigned lds, int i) const {
     const short *tile = base + (int64_t)row0 * stride;
-    if (LP == DP || active)
+    if (ALL_ACTIVE || active)
       load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (unsigned)(i * NW + wave) * 1024u);
   }
 
@@ -379,7 +392,7 @@ struct TileLoader {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
       const int r = min(row0 + i * NW * RPL + row_in, nrows - 1);
-      if (LP == DP || active)
+      if (ALL_ACTIVE || active)
         load_lds_16(base + (int64_t)r * stride + chunk * 8, lds + (unsigned)(i * NW + wave) * 1024u);
     }
   }

@@ -290,7 +290,9 @@ struct HalfTag {
   static constexpr bool inner = INNER;
 };
 
-template <typename T, int DP, int BKV>
+// PAD: the head dimension is a multiple of 8 below DP; the columns beyond it are zeros in LDS and in
+// the register fragments, and are not stored.
+template <typename T, int DP, int BKV, bool PAD>
 __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const FwdParams p) {
   using L = FwdDirectLayout<DP, BKV>;
   constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
@@ -321,7 +323,8 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   short *O = (short *)p.o.ptr + b * p.o.stride_batch + hd * p.o.stride_head;
   float *LSE = p.lse + (int64_t)bh * p.seqlen_q_rounded;
 
-  const TileLoader<DP, BKV, kFwdWaves> kload(K, p.k.stride_seq), vload(V, p.v.stride_seq);
+  const int hdim = PAD ? p.headdim : DP;
+  const TileLoader<DP, BKV, kFwdWaves, PAD> kload(K, p.k.stride_seq, hdim / 8), vload(V, p.v.stride_seq, hdim / 8);
   const int seqlen_k = p.seqlen_k;
   const float scale_log2 = p.scale_log2;
 
@@ -334,6 +337,10 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   const int n_inside = seqlen_k / BKV;  // tiles whose every row exists
 
   const unsigned lds_base = lds_u32(smem);  // LDS byte address of smem
+  if (PAD) {
+    zero_lds<NTHREADS>(smem, L::STAGE_ELEMS);
+    __syncthreads();
+  }
   auto issue_k = [&](int t) {
     const unsigned dst = lds_base + 2u * (unsigned)(L::K_BASE + (t % L::K_STAGES) * L::TILE_ELEMS);
     if (t < n_inside) kload.issue(t * BKV, dst); else kload.issue_clamped(t * BKV, seqlen_k, dst);
@@ -354,7 +361,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
     const bool ok = row < p.seqlen_q;
     const short *rp = Q + (int64_t)row * p.q.stride_seq;
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[ks] = load_chunk(rp, 16 * ks + 8 * h, DP, ok, true);
+    for (int ks = 0; ks < KS; ks++) qf[ks] = load_chunk(rp, 16 * ks + 8 * h, hdim, ok, true);
   }
 
   // Fragment addresses (swizzled, 32-bit LDS pointers).  kcur points into the stage of the K tile
@@ -458,7 +465,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   // time between the units of tile t's first step.  Issued back to back by all waves at once they
   // queue up in the memory pipeline, and a wave whose load cannot issue cannot issue its MFMAs
   // either.
-  constexpr int LOADS = TileLoader<DP, BKV, kFwdWaves>::LOADS;
+  constexpr int LOADS = TileLoader<DP, BKV, kFwdWaves, PAD>::LOADS;
   constexpr int LOAD_EVERY = KS / LOADS;
   auto step = [&](int j, auto half_tag, auto spread_tag) {
     constexpr int HALF = decltype(half_tag)::value;
@@ -585,7 +592,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const Fwd
   // The patch overlays the stages; the loop's last barrier already ordered it after all reads.
   short *patch = smem + wave * 32 * (DP + 8);
   store_transposed_acc<T, DP>(oacc, inv_l, patch, O + (int64_t)q0w * p.o.stride_seq,
-                              p.o.stride_seq, p.seqlen_q - q0w, DP, true);
+                              p.o.stride_seq, p.seqlen_q - q0w, hdim, true);
 }
 
 }  // namespace fa2

@@ -17,16 +17,24 @@ void launch_generic(int dp, const FwdParams &p, dim3 grid, dim3 block, hipStream
   }
 }
 
+template <typename T, bool PAD>
+void launch_direct(int dp, const FwdParams &p, dim3 grid, dim3 block, hipStream_t s) {
+  switch (dp) {
+    case 32: hipLaunchKernelGGL((fwd_direct_kernel<T, 32, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
+    case 64: hipLaunchKernelGGL((fwd_direct_kernel<T, 64, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
+    case 96: hipLaunchKernelGGL((fwd_direct_kernel<T, 96, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fwd_direct_kernel<T, 128, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
+  }
+}
+
 template <typename T>
 void launch(int dp, const FwdParams &p, dim3 grid, hipStream_t s) {
   const dim3 block(64 * kFwdWaves);
   if (fwd_direct_ok(dp, p)) {
-    switch (dp) {
-      case 32: hipLaunchKernelGGL((fwd_direct_kernel<T, 32, kFwdBlockKV>), grid, block, 0, s, p); break;
-      case 64: hipLaunchKernelGGL((fwd_direct_kernel<T, 64, kFwdBlockKV>), grid, block, 0, s, p); break;
-      case 96: hipLaunchKernelGGL((fwd_direct_kernel<T, 96, kFwdBlockKV>), grid, block, 0, s, p); break;
-      default: hipLaunchKernelGGL((fwd_direct_kernel<T, 128, kFwdBlockKV>), grid, block, 0, s, p); break;
-    }
+    if (p.headdim == dp)
+      launch_direct<T, false>(dp, p, grid, block, s);
+    else
+      launch_direct<T, true>(dp, p, grid, block, s);
     return;
   }
   if (p.vec)

@@ -65,7 +65,7 @@ SMALL_CASES = [
     (2, 4, 512, 512, 64, torch.float16, 1.0),
     (1, 2, 75, 75, 64, torch.float16, 1.0),       # shorter than one tile
     (1, 2, 300, 300, 128, torch.bfloat16, 1.0),   # ragged tail
-    (2, 3, 333, 200, 48, torch.float16, 1.0),     # more queries than keys, padded head dim
+    (2, 3, 333, 200, 48, torch.float16, 1.0),     # more queries than keys, head dim padded to 64
     (2, 3, 200, 333, 96, torch.bfloat16, 1.0),    # more keys than queries
     (1, 2, 130, 130, 32, torch.float16, 1.0),
     (1, 2, 100, 100, 40, torch.bfloat16, 1.0),    # head dim multiple of 8 but not of 16
@@ -79,6 +79,14 @@ SMALL_CASES = [
     (1, 2, 333, 200, 192, torch.float16, 1.0),
     (2, 2, 300, 300, 256, torch.bfloat16, 1.0),
     (1, 1, 130, 130, 250, torch.float16, 1.0),    # above 128 and not a multiple of 8
+    # head dims that are a multiple of 8 below the table row's: the padded LDS-direct kernels
+    (2, 2, 333, 333, 8, torch.float16, 1.0),
+    (1, 2, 200, 450, 24, torch.bfloat16, 1.0),
+    (2, 2, 450, 200, 56, torch.float16, 1.0),
+    (1, 2, 333, 333, 72, torch.bfloat16, 1.0),
+    (2, 2, 200, 450, 88, torch.float16, 1.0),
+    (1, 2, 333, 333, 104, torch.bfloat16, 1.0),
+    (1, 2, 450, 200, 120, torch.float16, 1.0),
 ]
 
 
