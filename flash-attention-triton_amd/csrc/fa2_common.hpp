@@ -279,6 +279,8 @@ __device__ __forceinline__ unsigned lds_u32(const short *p) {
       (int)(unsigned)(uintptr_t)(__attribute__((address_space(3))) const void *)p);
 }
 __device__ __forceinline__ void load_lds_16(const short *gsrc, unsigned lds_wave_addr) {
+  // State the uniformity the "s" constraint needs (folds away when the value is already scalar).
+  lds_wave_addr = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_wave_addr);
   asm volatile(
       "s_mov_b32 m0, %1\n\t"
       "s_nop 0\n\t"
@@ -297,6 +299,7 @@ __device__ __forceinline__ void load_lds_16(const short *uniform_base, unsigned 
   const uint64_t lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)raw);
   const uint64_t ubase = (hi << 32) | lo;
   uniform_base = (const short *)(uintptr_t)ubase;
+  lds_wave_addr = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_wave_addr);
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
       "s_nop 0\n\t"
