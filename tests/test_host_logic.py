@@ -198,6 +198,28 @@ def test_launcher_assertions_mirror_reference(fa2_module):
         fwd(q, q, q, None, *tail)
 
 
+def test_cpp_autograd_node_is_built_and_matches_the_library(capi, fa2_module):
+    """The C++ autograd node (csrc/fa2_torch_autograd.cpp) loads without a GPU, is linked against
+    the same ABI as the ctypes binding, and is what the public functions record."""
+    node = fa2_module._cpp_node()
+    assert node is not None, "flash-attention-triton_amd/_fa2_torch.so is not built (python flash-attention-triton_amd/build.py)"
+    assert node.abi_version() == capi.ABI_VERSION
+    q = torch.zeros(1, 2, 8, 16, dtype=torch.float16)
+    with pytest.raises(AssertionError, match="must reside on CUDA device"):  # the launcher's checks come first
+        fa2_module._apply(q, q, q, None, fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC)
+
+
+def test_noalloc_entry_point_refuses_sizes_beyond_its_scratch(capi):
+    """The size check of fa2_bwd_fused_noalloc comes before anything touches a device."""
+    lib = capi.load()
+    n_r = 1024
+    b = capi.FA2_NOALLOC_MAX_ROWS // n_r + 1
+    args = [16] * 9 + [b, 1, n_r, n_r, 64, n_r] + [0] * 24 + [0.125, capi.FA2_DTYPE_F16, 0, capi.FA2_CONFIG_AUTO, None]
+    status = lib.fa2_bwd_fused_noalloc(*args)
+    assert lib.fa2_status_string(status) == b"FA2_ERR_TOO_LARGE"
+    assert b"FA2_NOALLOC_MAX_ROWS" in lib.fa2_last_error_string()
+
+
 def test_workload_table_matches_baseline(workloads):
     w = workloads.WORKLOADS
     assert w["C1"].shape == (2, 4, 512, 64) and w["C1"].dtype == torch.float16

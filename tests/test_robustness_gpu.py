@@ -80,6 +80,31 @@ def test_ragged_shapes_on_fast_kernels(fa, case, deterministic):
         _assert_close(name, g, w)
 
 
+# ---------------------------------------------------------------- the two autograd nodes
+@pytest.mark.parametrize("case", [(2, 3, 333, 200, 64, torch.float16, None), (1, 2, 640, 640, 128, torch.bfloat16, 0.2),
+                                  (1, 2, 300, 300, 96, torch.float32, None), (1, 2, 257, 257, 64, torch.bfloat16, -0.125)],
+                         ids=["f16", "bf16-scale", "f32-input", "negative-scale"])
+def test_cpp_autograd_node_equals_python_class(fa, fa2_module, case):
+    """The public function records the C++ node (csrc/fa2_torch_autograd.cpp); the reference-shaped
+    Python class FlashAttentionV2Function makes the same launches: outputs and gradients are equal
+    bit for bit, input casts and a negative scale included."""
+    b, h, nq, nk, d, dtype, scale = case
+    assert fa2_module._cpp_node() is not None, "_fa2_torch.so is not built"
+    q, k, v, d_o = _seeded((b, h, nq, d), (b, h, nk, d), dtype)
+    cfg = fa2_module.GFX950_KERNEL_CONFIG_NON_DETERMINISTIC
+    results = []
+    for use_class in (False, True):
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        out = (fa2_module.FlashAttentionV2Function.apply(qg, kg, vg, scale, cfg) if use_class
+               else fa.flash_attention_v2(qg, kg, vg, scale, False))
+        out.backward(d_o.cuda())
+        torch.cuda.synchronize()
+        results.append((out.detach(), qg.grad, kg.grad, vg.grad))
+    for name, a, c in zip(("o", "dq", "dk", "dv"), *results):
+        assert a.dtype == c.dtype == dtype, name
+        assert torch.equal(a, c), f"{name} differs between the C++ node and the Python class"
+
+
 # ---------------------------------------------------------------- seeded randomised sweep
 def test_randomised_shape_sweep(fa):
     """48 seeded cases of mixed head dimension, Nq != Nk, dtype and mode against the oracle's formula
