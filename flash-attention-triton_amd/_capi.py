@@ -15,7 +15,7 @@ import threading
 # The in-tree build; FA2_GFX950_LIBRARY names another build of the same ABI (e.g. one under test).
 LIBRARY_PATH = pathlib.Path(os.environ.get("FA2_GFX950_LIBRARY") or
                             pathlib.Path(__file__).resolve().parent / "csrc" / "libfa2_gfx950.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 FA2_DTYPE_F16 = 0
 FA2_DTYPE_BF16 = 1
@@ -35,7 +35,7 @@ class ConfigInfo(ctypes.Structure):
         "bwd_block_q", "bwd_block_kv", "bwd_waves",
         "dq_block_q", "dq_block_kv", "dq_waves",
         "lds_direct", "fwd_wg_per_cu", "dq_wg_per_cu", "dkdv_wg_per_cu",
-        "lds_stages", "dkdv_passes", "head_group")]
+        "lds_stages", "dkdv_passes", "head_group", "dq_atomic")]
 
     def as_dict(self) -> dict:
         return {name: getattr(self, name) for name, _ in self._fields_}

@@ -5,9 +5,11 @@ Mirrors ``KernelsConfigV2`` and ``init_to_zero_v2`` of the reference
 ``flash_attention_v2_custom`` keeps working, without importing Triton.  The fields keep their
 names.  The tile shapes of the gfx950 kernels are compiled into ``libfa2_gfx950.so`` (one table row
 per padded head dimension, chosen by the library from the problem), so of the fields below only
-``max_headdim`` (largest accepted head dimension, padding of the log-sum-exp rows) and the
-``SEQUENCE_PARALLEL`` flag of the backward configurations (which backward mode is requested) have
-an effect; the Triton tile, warp and stage counts are accepted and ignored.  The reference's
+``max_headdim`` (largest accepted head dimension, padding of the log-sum-exp rows), the
+``SEQUENCE_PARALLEL`` flag of the backward configurations (which backward mode is requested) and,
+next to it, ``ATOMIC_DQ`` (run the reference's atomic-add formulation of that mode, see
+``KernelsConfigV2.atomic_dq``) have an effect; the Triton tile, warp and stage counts are accepted
+and ignored.  The reference's
 kernel-cache key helpers (_configurators_v2.py:40-78) have no counterpart: there is no run-time
 compilation and therefore no kernel cache to key.
 """
@@ -26,9 +28,9 @@ class BackwardConfig:
     """Stand-in for ``triton.Config`` in ``backward_autotune_configs``.
 
     Any object with the same attributes (``kwargs``, ``num_warps``, ``num_stages``,
-    ``pre_hook``) is accepted, a real ``triton.Config`` included.  Only
-    ``kwargs["SEQUENCE_PARALLEL"]`` changes behaviour: it selects the non-deterministic
-    backward (reference: flash_attention_2.py:204-207, _triton_kernels_v2.py:466-525).
+    ``pre_hook``) is accepted, a real ``triton.Config`` included.  ``kwargs["SEQUENCE_PARALLEL"]``
+    selects the non-deterministic backward (reference: flash_attention_2.py:204-207,
+    _triton_kernels_v2.py:466-525); ``kwargs["ATOMIC_DQ"]`` beside it selects how that mode is run.
     """
 
     kwargs: dict[str, Any]
@@ -75,6 +77,21 @@ class KernelsConfigV2:
         """True unless a backward configuration asks for sequence-parallel dQ accumulation."""
         return not any(bool(getattr(c, "kwargs", {}).get("SEQUENCE_PARALLEL", False))
                        for c in self.backward_autotune_configs)
+
+    @property
+    def atomic_dq(self) -> bool:
+        """True when a sequence-parallel backward configuration also sets ``ATOMIC_DQ``.
+
+        The non-deterministic mode then runs as the reference formulates it
+        (_triton_kernels_v2.py:336-339): one kernel per key tile that adds its dQ contributions into
+        an fp32 accumulator with global atomics.  Without the flag (the default table) the mode runs
+        the same two atomic-free kernels as the deterministic one, which on MI355X is two to three
+        times faster; the flag is there for callers who want the reference's accumulation order
+        semantics or want to measure it.  Head dimensions 32, 64 and 128 only.
+        """
+        return any(bool(getattr(c, "kwargs", {}).get("SEQUENCE_PARALLEL", False))
+                   and bool(getattr(c, "kwargs", {}).get("ATOMIC_DQ", False))
+                   for c in self.backward_autotune_configs)
 
 
 def init_to_zero_v2(name: str) -> Callable[[dict[str, torch.Tensor]], torch.Tensor]:

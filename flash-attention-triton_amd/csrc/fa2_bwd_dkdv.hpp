@@ -282,16 +282,34 @@ struct DkvDirectLayout {
 
 // PAD: the head dimension is a multiple of 8 below DP; the columns beyond it are zeros in LDS and in
 // the register fragments, and are not stored.
-template <typename T, int DP, int BQ, bool PAD>
-__global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_direct_kernel(const BwdParams p) {
+//
+// ATOMIC_DQ: the kernel is the whole backward of the reference's sequence-parallel mode
+// (_triton_kernels_v2.py:336-339, 466-494): besides dK and dV of its key tile it forms, for every
+// 32-row query block, the block's contribution dS K to dQ (a fifth GEMM) and adds it with fp32
+// global atomics into p.dq_accum, which the caller zeroed and converts afterwards.  dS has the key
+// index across lanes, the contraction index of that GEMM, so it travels through LDS: every wave
+// writes its 32 key rows of dS ([key][query], two buffers used alternately), the workgroup meets at
+// a barrier, and wave w multiplies column block w % DB of K by the dS rows of key group w / DB
+// (at DB = 4: 32 of the 128 columns each, all 128 keys).  The result leaves the MFMA with the head
+// dimension across lanes, so every atomic instruction covers two 128-byte row segments.
+template <typename T, int DP, int BQ, bool PAD, bool ATOMIC_DQ = false>
+__global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 && !ATOMIC_DQ ? 2 : 1)) void bwd_dkdv_direct_kernel(const BwdParams p) {
   using L = DkvDirectLayout<DP, BQ>;
   constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
   constexpr int NTHREADS = 64 * kDkvWaves;
   static_assert(BQ == 64 && KS == 2 * DB, "schedule is written for 64-row query tiles of two blocks");
   static_assert(BQ <= NTHREADS, "one thread per row loads lse and delta");
   static_assert((L::STAGE_ELEMS * 2) % 256 == 0, "stages must start on a 256-byte LDS bank line");
+  static_assert(!ATOMIC_DQ || (kDkvWaves % DB == 0 && !PAD), "the dQ GEMM splits column blocks evenly over the waves");
+  // dS exchange area: kDkvBlockKV key rows of 32 queries, pitch 36 halves (72 bytes: rows start on
+  // 8-byte words and fall on different banks), two buffers.
+  constexpr int DS_PITCH = 36;
+  constexpr int DS_BUF_ELEMS = kDkvBlockKV * DS_PITCH;
+  constexpr int DS_BASE = (L::TOTAL_ELEMS + 7) / 8 * 8;
+  constexpr int KG = ATOMIC_DQ ? kDkvBlockKV * DB / kDkvWaves : 32;  // keys a wave contracts over in the dQ GEMM
+  constexpr int KSQ = KG / 16;                                        // its MFMAs per block
 
-  __shared__ __attribute__((aligned(1024))) short smem[L::TOTAL_ELEMS];
+  __shared__ __attribute__((aligned(1024))) short smem[ATOMIC_DQ ? DS_BASE + 2 * DS_BUF_ELEMS : L::TOTAL_ELEMS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -344,28 +362,37 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       gload.issue_clamped(row0, seqlen_q, dst + 2u * L::TILE_ELEMS);
     }
   };
-  // lse*log2e and delta of a tile go through registers into the stage's statistics area (rows
-  // beyond the sequence get 0: their probabilities are zeroed by the row mask).
+  // lse and delta of a tile go through registers into the stage's statistics area.  load_stats
+  // only issues the two loads: any arithmetic on a loaded value makes the wave wait for it on the
+  // spot (and, loads returning in order, for every tile load issued before it), once per tile and
+  // with nothing else to run on the SIMD.  The values are first touched a tile later, in
+  // store_stats.  Rows beyond the sequence take the last row's values (finite; the row mask zeroes
+  // their probabilities).
   float lse_reg = 0.f, delta_reg = 0.f;
   auto load_stats = [&](int t) {
     if (tid < BQ) {
-      const int row = q_begin + t * BQ + tid;
-      const bool ok = row < seqlen_q;
-      lse_reg = ok ? LSE[row] * kLog2e : 0.f;
-      delta_reg = ok ? DELTA[row] : 0.f;
+      const int row = min(q_begin + t * BQ + tid, seqlen_q - 1);
+      lse_reg = LSE[row];
+      delta_reg = DELTA[row];
     }
   };
   auto store_stats = [&](int t) {
     float *sl = reinterpret_cast<float *>(smem + (t % L::STAGES) * L::STAGE_ELEMS + 2 * L::TILE_ELEMS);
+    // The compiler's own wait for the two loads counts the atomics issued since as if everything
+    // completed in order; atomics complete ahead of older loads.
+    if (ATOMIC_DQ) wait_vmem_all();
     if (tid < BQ) {
-      sl[tid] = lse_reg;
+      sl[tid] = lse_reg * kLog2e;
       sl[BQ + tid] = -delta_reg;  // negated: it is the accumulator the dP MFMAs start from
     }
   };
-  // Prologue: the first tile and this wave's K and V rows are requested before anything waits;
-  // tiles 1 and 2 follow right after the first barrier and land while tile 0 is being multiplied,
-  // so the first MFMA waits for one tile, not three.
-  if (0 < n_tiles) issue_tile(0);
+  // Prologue: every global load of the first three tiles and of this wave's K and V rows is
+  // issued before anything waits, so that the workgroup pays one memory latency, not one per
+  // tile.  (Tiles 1 and 2 cannot be requested later: the second block of tile 0 already fetches
+  // the first fragments of tile 1.)
+#pragma unroll
+  for (int t = 0; t < L::STAGES; t++)
+    if (t < n_tiles) issue_tile(t);
 
   // B operands: lane (c, h) holds row kv0w + c of K and of V, columns 16 ks + 8 h + j.
   s16x8 kf[KS], vf[KS];
@@ -380,6 +407,24 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       vf[ks] = load_chunk(vp, 16 * ks + 8 * h, hdim, ok, true);
     }
   }
+  // B operands of the dQ GEMM: lane (c, h) holds column 32 (wave % DB) + c of K for the keys of key
+  // group wave / DB, element j of k-step s being key 16 s + 8 (j / 4) + 4 h + j % 4 of the group (the
+  // order in which the transposing LDS reads deliver the dS rows).
+  s16x8 kb[KSQ];
+  float *dq_rows = nullptr;  // this lane's column of the fp32 dQ accumulator, row 4 h of the sequence
+  if (ATOMIC_DQ) {
+    const int col = 32 * (wave % DB) + c;
+    const int key0 = kv0 + (wave / DB) * KG;
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ks++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const int key = key0 + 16 * ks + 8 * (j >> 2) + 4 * h + (j & 3);
+        kb[ks][j] = key < p.seqlen_k ? K[(int64_t)key * p.k.stride_seq + col] : (short)0;
+      }
+    dq_rows = p.dq_accum + ((int64_t)bh * p.dq_accum_rows + 4 * h) * DP + col;
+  }
+
   // Statistics of the first three tiles: loaded now, written to LDS just before the first
   // barrier (the write has to wait for every load above, and the set-up below should not).
   float l3[L::STAGES], d3[L::STAGES];
@@ -434,9 +479,6 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   }
   wait_vmem_all();
   __syncthreads();
-#pragma unroll
-  for (int t = 1; t < L::STAGES; t++)
-    if (t < n_tiles) issue_tile(t);
   // Two rings of A fragments, preloaded with the Q rows and the dO rows of block 0.
   s16x8 ring[KS], ringb[KS];
 #pragma unroll
@@ -538,6 +580,17 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
     f32x8 dlo = {ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]};
     f32x8 dhi = {ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]};
     const s16x8 dsf[2] = {Elem<T>::pack8(dlo), Elem<T>::pack8(dhi)};
+    if (ATOMIC_DQ) {
+      // This lane's key row of dS: element j of dsf[t] is query 16 t + 8 (j / 4) + 4 h + j % 4.
+      short *row = smem + DS_BASE + HALF * DS_BUF_ELEMS + (32 * wave + c) * DS_PITCH + 4 * h;
+#pragma unroll
+      for (int t2 = 0; t2 < 2; t2++)
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+          const s16x4 w4 = {dsf[t2][4 * g], dsf[t2][4 * g + 1], dsf[t2][4 * g + 2], dsf[t2][4 * g + 3]};
+          *reinterpret_cast<s16x4 *>(row + 16 * t2 + 8 * g) = w4;
+        }
+    }
     // ---- dK^T += Q^T dS (ringb: Q^T -> dO rows of the next block) ------------------------------
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
@@ -545,6 +598,26 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
       spread_load(3 * KS + ks);
       ringb[ks] = lds_read_128(qnext[ks] + L::TILE_ELEMS + (HALF == 0 ? 32 * LP : 0));
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (ATOMIC_DQ) {
+      // ---- dQ[block] += dS K: every wave's dS rows are in LDS after this barrier (the buffer of
+      // the block before is being read by nobody: all waves passed that block's barrier) --------
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      const short *frag = smem + DS_BASE + HALF * DS_BUF_ELEMS +
+                          ((wave / DB) * KG + 4 * h + (i16 >> 2)) * DS_PITCH + 16 * g2 + 4 * (i16 & 3);
+      f32x16 dqb = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KSQ; ks++) {
+        const s16x8 a = lds_read_tr_frag(frag + 16 * ks * DS_PITCH, DS_PITCH);
+        dqb = Elem<T>::mfma(a, kb[ks], dqb);
+      }
+      // Element i is query row qb + 4 h + 8 (i / 4) + i % 4, this lane's column.  Rows up to the end
+      // of the last 64-row tile exist in the accumulator; masked rows add zeros.
+      float *dst = dq_rows + (int64_t)qb * DP;
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        __builtin_amdgcn_global_atomic_fadd_f32(
+            (__attribute__((address_space(1))) float *)(dst + (8 * (i >> 2) + (i & 3)) * DP), dqb[i]);
     }
   };
 
@@ -592,6 +665,35 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 ? 2 : 1)) void bwd_dkdv_d
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   store_transposed_acc<T, DP>(dkacc, p.scale, patch, DK + (int64_t)kv0w * p.dk.stride_seq,
                               p.dk.stride_seq, p.seqlen_k - kv0w, hdim, true);
+}
+
+// ---- fp32 dQ accumulator of the sequence-parallel mode ------------------------------------------
+// Cleared by a kernel, not a memset node, so that callers may capture the backward in a HIP graph.
+__global__ __launch_bounds__(256) void dq_accum_zero_kernel(float *acc, int64_t n4) {
+  const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256)
+    reinterpret_cast<f32x4 *>(acc)[i] = z;
+}
+
+// dq = scale * accumulator, rounded once to the tensor's type (the reference's dq.copy_(dq_accum),
+// flash_attention_2.py:277, with the scale the kernel left out).  One thread per 8 columns.
+template <typename T>
+__global__ __launch_bounds__(256) void dq_accum_convert_kernel(const BwdParams p) {
+  const int cpr = p.headdim / 8;  // headdim is a multiple of 32 in this mode
+  const int64_t total = (int64_t)p.batch * p.nheads * p.seqlen_q * cpr;
+  for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x; id < total; id += (int64_t)gridDim.x * 256) {
+    const int cc = (int)(id % cpr);
+    const int64_t r = id / cpr;
+    const int row = (int)(r % p.seqlen_q);
+    const int bh = (int)(r / p.seqlen_q);
+    const int b = bh / p.nheads, hd = bh % p.nheads;
+    const float *src = p.dq_accum + ((int64_t)bh * p.dq_accum_rows + row) * p.headdim + cc * 8;
+    const f32x4 lo = *reinterpret_cast<const f32x4 *>(src), hi = *reinterpret_cast<const f32x4 *>(src + 4);
+    const f32x8 x = {lo[0] * p.scale, lo[1] * p.scale, lo[2] * p.scale, lo[3] * p.scale,
+                     hi[0] * p.scale, hi[1] * p.scale, hi[2] * p.scale, hi[3] * p.scale};
+    short *dst = (short *)p.dq.ptr + b * p.dq.stride_batch + hd * p.dq.stride_head + (int64_t)row * p.dq.stride_seq + cc * 8;
+    *reinterpret_cast<s16x8 *>(dst) = Elem<T>::pack8(x);
+  }
 }
 
 }  // namespace fa2

@@ -41,12 +41,20 @@ constexpr int kHeadGroup = 64;  // (batch, head) pairs dispatched together: 8 pe
 
 const fa2_config_info kTable[] = {
     // id DP  fwd:BQ       BKV        waves dK/dV:BQ   BKV       waves dQ:BQ    BKV      waves fast fwd/CU dq/CU dkdv/CU stages passes group
-    {0, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 4, 3, 3, 1, kHeadGroup},
-    {1, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 3, 2, 3, 1, kHeadGroup},
-    {2, 96, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup},
-    {3, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup},
-    {4, 192, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 1, kHeadGroup},
-    {5, 256, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 2, kHeadGroup},
+    {0, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 4, 3, 3, 1, kHeadGroup, 0},
+    {1, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 3, 2, 3, 1, kHeadGroup, 0},
+    {2, 96, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup, 0},
+    {3, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup, 0},
+    {4, 192, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 1, kHeadGroup, 0},
+    {5, 256, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 2, kHeadGroup, 0},
+    // Sequence-parallel rows (dq_atomic = 1): the backward is one key-tile-parallel kernel that adds its
+    // dQ contributions into an fp32 workspace with global atomics, the reference's non-deterministic
+    // formulation (_triton_kernels_v2.py:336-339).  Never picked automatically: on MI355X the atomics
+    // alone take longer than the whole two-kernel backward (profiles/bwd_sequence_parallel_atomic_*.txt);
+    // a caller selects them by id.  Forward columns as in the row of the same head dimension.
+    {6, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 0, 1, 3, 1, kHeadGroup, 1},
+    {7, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 0, 1, 3, 1, kHeadGroup, 1},
+    {8, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 0, 1, 3, 1, kHeadGroup, 1},
 };
 constexpr int kTableRows = sizeof(kTable) / sizeof(kTable[0]);
 
@@ -62,9 +70,12 @@ int head_group(int cfg, int64_t heads) {
 
 int pick_config(int headdim) {
   for (int i = 0; i < kTableRows; i++)
-    if (headdim <= kTable[i].headdim_padded) return i;
+    if (!kTable[i].dq_atomic && headdim <= kTable[i].headdim_padded) return i;
   return -1;
 }
+
+// Query rows of the fp32 dQ accumulator of a sequence-parallel row: whole 64-row query tiles.
+int64_t dq_accum_rows(int seqlen_q) { return ((int64_t)seqlen_q + kDkvBlockQ - 1) / kDkvBlockQ * kDkvBlockQ; }
 
 int resolve_config(int config_id, int headdim, int *out) {
   if (config_id == FA2_CONFIG_AUTO) {
@@ -75,6 +86,9 @@ int resolve_config(int config_id, int headdim, int *out) {
     return fail(FA2_ERR_BAD_CONFIG, "config id %d outside the table [0, %d)", config_id, kTableRows);
   if (kTable[config_id].headdim_padded < headdim)
     return fail(FA2_ERR_BAD_CONFIG, "config %d is built for headdim <= %d, got %d", config_id,
+                kTable[config_id].headdim_padded, headdim);
+  if (kTable[config_id].dq_atomic && kTable[config_id].headdim_padded != headdim)
+    return fail(FA2_ERR_BAD_CONFIG, "sequence-parallel config %d is built for headdim == %d, got %d", config_id,
                 kTable[config_id].headdim_padded, headdim);
   *out = config_id;
   return FA2_OK;
@@ -182,8 +196,9 @@ int preprocess_impl(const fa2_tensor &o, const fa2_tensor &d_o, float *delta, in
 
 // Backward behind fa2_bwd, fa2_bwd_fused and fa2_bwd_packed.  With a.o given, delta is an
 // output: it is formed by the dQ kernel when the fast dQ kernel applies (and the dK/dV kernel then
-// runs second), otherwise by the preprocess kernel launched from here.  `deterministic` and
-// `workspace` are accepted and not needed: dQ is written once, in a fixed order, in both modes.
+// runs second), otherwise by the preprocess kernel launched from here.  With the rows the table
+// picks by itself `deterministic` and `workspace` are accepted and not needed: dQ is written once,
+// in a fixed order, in both modes.  The sequence-parallel rows (dq_atomic) take the workspace.
 int bwd_impl(const fa2_bwd_args &a, void *stream) {
   int rc = check_common(a.batch, a.nheads, a.seqlen_q, a.seqlen_k, a.headdim, a.seqlen_q_rounded, a.dtype);
   if (rc) return rc;
@@ -238,6 +253,8 @@ int bwd_impl(const fa2_bwd_args &a, void *stream) {
   const bool bf16 = a.dtype == FA2_DTYPE_BF16;
   const int dp = kTable[cfg].headdim_padded;
   const int64_t bh = (int64_t)a.batch * a.nheads;
+  p.dq_accum = nullptr;
+  p.dq_accum_rows = 0;
 
   fa2::BwdParams pk = p, pq = p;
   // The dK/dV kernel keeps the table's group size at every head count: with one or two workgroups
@@ -253,6 +270,34 @@ int bwd_impl(const fa2_bwd_args &a, void *stream) {
     fa2::launch_dkdv(bf16, dp, pk, dim3((unsigned)nwg_k), s);
     return launch_status("backward dK/dV launch");
   };
+
+  if (kTable[cfg].dq_atomic) {
+    // Sequence-parallel mode: clear the accumulator, (form delta), one key-tile-parallel kernel for
+    // dK, dV and the atomic dQ contributions, then dq = scale * accumulator.
+    if (a.deterministic)
+      return fail(FA2_ERR_BAD_CONFIG, "config %d accumulates dQ with atomics: not available with deterministic=1", cfg);
+    if (!(want_dq && want_dkdv))
+      return fail(FA2_ERR_NULL_POINTER, "the sequence-parallel backward produces dq, dk and dv together");
+    if (a.workspace == nullptr)
+      return fail(FA2_ERR_WORKSPACE, "config %d needs fa2_bwd_workspace_bytes() bytes of workspace", cfg);
+    if (reinterpret_cast<uintptr_t>(a.workspace) % 16 != 0)
+      return fail(FA2_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+    if (!fa2::seqpar_atomic_ok(dp, pk))
+      return fail(FA2_ERR_BAD_CONFIG, "the sequence-parallel kernels need 16-byte aligned tensors and strides "
+                                      "and a head dimension of 32, 64 or 128");
+    pk.dq_accum = static_cast<float *>(a.workspace);
+    pk.dq_accum_rows = (int)dq_accum_rows(a.seqlen_q);
+    fa2::launch_dq_accum_zero(pk.dq_accum, bh * pk.dq_accum_rows * a.headdim, s);
+    if ((rc = launch_status("dQ accumulator clear"))) return rc;
+    if (fused) {
+      rc = preprocess_impl(a.o, a.d_o, a.delta, a.batch, a.nheads, a.seqlen_q, a.headdim, a.seqlen_q_rounded,
+                           a.dtype, stream);
+      if (rc) return rc;
+    }
+    if ((rc = run_dkdv())) return rc;
+    fa2::launch_dq_accum_convert(bf16, pk, s);
+    return launch_status("dQ accumulator convert");
+  }
 
   if (fused && fa2::dq_direct_ok(dp, pq) && vec_ok(p.o, a.headdim)) {
     // dQ first: it writes delta, which the dK/dV kernel reads.
@@ -396,10 +441,12 @@ int fa2_bwd_preprocess(const void *o, const void *d_o, float *delta, int batch, 
 
 size_t fa2_bwd_workspace_bytes(int batch, int nheads, int seqlen_q, int seqlen_k, int headdim,
                                int deterministic, int config_id) {
-  (void)batch; (void)nheads; (void)seqlen_q; (void)seqlen_k; (void)headdim;
-  (void)deterministic; (void)config_id;
-  // Both modes write dQ exactly once from registers: no accumulation buffer.
-  return 0;
+  (void)seqlen_k; (void)deterministic;
+  // The two-kernel backward writes dQ exactly once from registers: no accumulation buffer.  A
+  // sequence-parallel row accumulates dQ in fp32: batch * nheads * (seqlen_q rounded up to 64) * headdim floats.
+  if (config_id < 0 || config_id >= kTableRows || !kTable[config_id].dq_atomic) return 0;
+  if (batch <= 0 || nheads <= 0 || seqlen_q <= 0 || headdim <= 0) return 0;
+  return (size_t)batch * (size_t)nheads * (size_t)dq_accum_rows(seqlen_q) * (size_t)headdim * sizeof(float);
 }
 
 int fa2_bwd(const void *q, const void *k, const void *v, const void *d_o, const float *lse,

@@ -28,12 +28,20 @@ inline bool dq_direct_ok(int dp, const BwdParams &p) {
 inline bool dkdv_direct_ok(int dp, const BwdParams &p) {
   return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.q) && direct_stride_ok(p.d_o);
 }
+// The sequence-parallel (atomic dQ) kernels: the fast dK/dV kernel's conditions, a head dimension
+// of exactly 32, 64 or 128 and 16-byte aligned dq rows.
+inline bool seqpar_atomic_ok(int dp, const BwdParams &p) {
+  return dkdv_direct_ok(dp, p) && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128);
+}
 
 // bf16 != 0 selects the bf16 kernels, otherwise fp16.
 void launch_fwd(bool bf16, int dp, const FwdParams &p, dim3 grid, hipStream_t s);
 void launch_preprocess(bool bf16, const PreParams &p, dim3 grid, hipStream_t s);
 // fuse_delta: the fast dQ kernel also forms delta from O and dO (dq_direct_ok must hold).
 void launch_dq(bool bf16, int dp, const BwdParams &p, dim3 grid, bool fuse_delta, hipStream_t s);
+// With p.dq_accum set the sequence-parallel kernel runs: dK, dV and atomic dQ contributions.
 void launch_dkdv(bool bf16, int dp, const BwdParams &p, dim3 grid, hipStream_t s);
+void launch_dq_accum_zero(float *acc, int64_t floats, hipStream_t s);
+void launch_dq_accum_convert(bool bf16, const BwdParams &p, hipStream_t s);
 
 }  // namespace fa2

@@ -42,6 +42,11 @@ struct BwdParams {
   Tensor4 q, k, v, d_o, dq, dk, dv;
   Tensor4 o;         // only read by the dQ kernel when it also forms delta
   float *delta_out;  // where that kernel writes delta (the same buffer `delta` points to)
+  // Sequence-parallel mode only: fp32 (batch * nheads, dq_accum_rows, headdim) accumulator the
+  // key-tile kernel adds its dQ contributions to; dq_accum_rows is seqlen_q rounded up to the
+  // kernel's 64-row query tile.
+  float *dq_accum;
+  int dq_accum_rows;
   const float *lse;
   const float *delta;
   int batch, nheads, seqlen_q, seqlen_k, headdim, seqlen_q_rounded;

@@ -203,6 +203,7 @@ def _flash_attention_backward(
     delta = torch.empty_like(lse)
     softmax_scale = softmax_scale or 1.0 / math.sqrt(headdim)
     deterministic = 1 if kernels_config.deterministic else 0
+    config_id = _atomic_row(headdim) if kernels_config.atomic_dq else _capi.FA2_CONFIG_AUTO
 
     # Negative scale: run on -Q with |scale| (see the forward launcher); dK and dV are unchanged
     # and dQ comes out with the opposite sign.
@@ -212,9 +213,10 @@ def _flash_attention_backward(
 
     # Both launches of the reference launcher (preprocess, then the main kernel) in one call:
     # with `o` in the record the library forms delta on the way.  Every tensor is contiguous here
-    # (asserted above), so shapes, dtype, scale and mode identify the record; the workspace size
-    # is asked once per record (it is 0: dQ is written directly).
-    key = (q.shape, seqlen_k, q.dtype, softmax_scale, deterministic, threading.get_ident())
+    # (asserted above), so shapes, dtype, scale, mode and table row identify the record; the
+    # workspace size is asked once per record (0 unless a sequence-parallel row was asked for: dQ
+    # is written directly).
+    key = (q.shape, seqlen_k, q.dtype, softmax_scale, deterministic, config_id, threading.get_ident())
     cached = _BWD_ARGS.get(key)
     if cached is None:
         args = _capi.BwdArgs()
@@ -225,9 +227,9 @@ def _flash_attention_backward(
         args.batch, args.nheads, args.seqlen_q, args.seqlen_k = batch, nheads, seqlen_q, seqlen_k
         args.headdim, args.seqlen_q_rounded = headdim, seqlen_q_rounded
         args.softmax_scale, args.dtype = softmax_scale, _COMPUTE_DTYPES[q.dtype]
-        args.deterministic, args.config_id = deterministic, _capi.FA2_CONFIG_AUTO
+        args.deterministic, args.config_id = deterministic, config_id
         ws_bytes = _capi.load().fa2_bwd_workspace_bytes(batch, nheads, seqlen_q, seqlen_k, headdim,
-                                                        deterministic, _capi.FA2_CONFIG_AUTO)
+                                                        deterministic, config_id)
         cached = (args, ws_bytes)
         _remember(_BWD_ARGS, key, cached)
     args, ws_bytes = cached
@@ -245,6 +247,19 @@ def _flash_attention_backward(
         _capi.check(status, "fa2_bwd")
     if negated:
         dq.neg_()
+
+
+_ATOMIC_ROWS: dict[int, int] = {}
+
+
+def _atomic_row(headdim: int) -> int:
+    """Id of the sequence-parallel (atomic dQ) table row for this head dimension."""
+    if not _ATOMIC_ROWS:
+        _ATOMIC_ROWS.update({row["headdim_padded"]: row["id"] for row in _capi.config_table() if row["dq_atomic"]})
+    if headdim not in _ATOMIC_ROWS:
+        raise ValueError(f"ATOMIC_DQ: the sequence-parallel atomic kernels exist for head dimensions "
+                         f"{sorted(_ATOMIC_ROWS)}, got {headdim}")
+    return _ATOMIC_ROWS[headdim]
 
 
 def _compute_dtype(dtype: torch.dtype) -> torch.dtype:
@@ -293,8 +308,11 @@ class FlashAttentionV2Function(torch.autograd.Function):
         q, k, v, output, lse = ctx.saved_tensors
         kernels_config = ctx.kernels_config
 
-        # Like the reference (flash_attention_2.py:364) the backward is not differentiable.
-        with torch.inference_mode():
+        # Like the reference (flash_attention_2.py:364) the backward is not differentiable.  It runs
+        # under no_grad rather than the reference's inference_mode: gradients that are inference
+        # tensors cannot be accumulated in place (a second backward into the same .grad, or q, k and
+        # v being one tensor, raises "Inplace update to inference tensor").
+        with torch.no_grad():
             dq = torch.empty_like(q)
             dk = torch.empty_like(k)
             dv = torch.empty_like(v)
@@ -345,7 +363,7 @@ def _apply(q, k, v, softmax_scale, kernels_config):  # noqa: ANN001, ANN202
     checks are the launcher's, a negative scale is folded into the sign of q.
     """
     node = _cpp_node()
-    if node is None:
+    if node is None or kernels_config.atomic_dq:  # the C++ node always lets the table choose
         return FlashAttentionV2Function.apply(q, k, v, softmax_scale, kernels_config)
     initial_dtype = q.dtype
     compute_dtype = _compute_dtype(initial_dtype)
@@ -401,6 +419,29 @@ GFX950_KERNEL_CONFIG_NON_DETERMINISTIC = KernelsConfigV2(
     max_warps=4,
     num_stages=2,
     backward_autotune_configs=GFX950_BACKWARD_CONFIGS_NON_DETERMINISTIC,
+)
+
+# The non-deterministic mode run the reference's way: one backward kernel per key tile, dQ
+# accumulated with fp32 global atomics (KernelsConfigV2.atomic_dq).  Not in the table of defaults,
+# because it is slower than the configuration above; pass it to flash_attention_v2_custom.
+GFX950_BACKWARD_CONFIGS_SEQUENCE_PARALLEL_ATOMIC = [
+    BackwardConfig(
+        {"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": True, "ATOMIC_DQ": True},
+        num_warps=4,
+        num_stages=2,
+        pre_hook=init_to_zero_v2("DQ"),
+    ),
+]
+GFX950_KERNEL_CONFIG_SEQUENCE_PARALLEL_ATOMIC = KernelsConfigV2(
+    block_rows_size=128,
+    block_cols_size=64,
+    min_block_headdim=32,
+    max_headdim=_capi.FA2_MAX_HEADDIM,
+    seqlen_cache_divisor=32,
+    min_warps=4,
+    max_warps=4,
+    num_stages=2,
+    backward_autotune_configs=GFX950_BACKWARD_CONFIGS_SEQUENCE_PARALLEL_ATOMIC,
 )
 
 _GPU_ARCHITECTURES = {
@@ -503,8 +544,9 @@ def flash_attention_v2_custom(
     Same contract as the reference (flash_attention_2.py:700-790): the dictionary is keyed by
     ``torch.cuda.get_device_capability()`` of the current device ((9, 5) on MI355X); a missing
     key raises ValueError.  Of the configuration, ``max_headdim`` and the ``SEQUENCE_PARALLEL``
-    flag of the backward configurations are honoured; the Triton tile, warp and stage counts are
-    accepted and ignored (the reference hands them to its kernels, flash_attention_2.py:137-141;
+    and ``ATOMIC_DQ`` flags of the backward configurations are honoured (the latter selects the
+    atomic-add backward, ``GFX950_KERNEL_CONFIG_SEQUENCE_PARALLEL_ATOMIC``); the Triton tile, warp
+    and stage counts are accepted and ignored (the reference hands them to its kernels, flash_attention_2.py:137-141;
     here the tile shapes are compiled in, one table row per padded head dimension).
 
     Example:

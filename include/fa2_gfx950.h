@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define FA2_ABI_VERSION 3
+#define FA2_ABI_VERSION 4
 
 /* Largest head dimension the kernels accept (the table's `max_headdim`). */
 #define FA2_MAX_HEADDIM 256
@@ -85,6 +85,8 @@ typedef struct fa2_config_info {
   int lds_stages;     /* LDS stages of the streamed operand in the kernels of this row */
   int dkdv_passes;    /* passes of the dK/dV kernel over the query tiles (2: half the columns each) */
   int head_group;     /* (batch, head) pairs dispatched together; head_group / 8 share one XCD's L2 */
+  int dq_atomic;      /* 1: sequence-parallel row - one backward kernel, dQ accumulated with fp32 global atomics
+                         in a workspace (never picked by FA2_CONFIG_AUTO; selected by id) */
 } fa2_config_info;
 
 /* One (batch, nheads, seqlen, headdim) tensor: device pointer and strides in elements. */
@@ -178,8 +180,11 @@ int fa2_bwd_preprocess(const void *o, const void *d_o, float *delta,
                        int dtype, void *stream);
 
 /*
- * Bytes of workspace the backward needs: 0, because dQ is written directly in both modes.
- * Stands in for the reference's dq_accum allocation (flash_attention_2.py:196).
+ * Bytes of workspace the backward needs.  Stands in for the reference's dq_accum allocation
+ * (flash_attention_2.py:196).  0 for FA2_CONFIG_AUTO and every row it can pick (dQ is written
+ * directly); for a sequence-parallel row (dq_atomic) the fp32 dQ accumulator:
+ * batch * nheads * ceil(seqlen_q / 64) * 64 * headdim * 4 bytes, 16-byte aligned, which the
+ * library clears itself on every call.
  */
 size_t fa2_bwd_workspace_bytes(int batch, int nheads, int seqlen_q, int seqlen_k, int headdim,
                                int deterministic, int config_id);
@@ -189,16 +194,21 @@ size_t fa2_bwd_workspace_bytes(int batch, int nheads, int seqlen_q, int seqlen_k
  * Replaces _flash_attention_backward's main launch, the dQ zero-fill pre-hook and the final
  * dq.copy_(dq_accum) (flash_attention_2.py:235-277, _configurators_v2.py:81-93,
  * _triton_kernels_v2.py:192-529).
- * Both values of `deterministic` run the same two kernels: a key-tile-parallel kernel for dK and
- * dV and a query-tile-parallel kernel that accumulates dQ in registers in a fixed order and writes
- * it once.  There are no atomics in either mode, so results are bit-identical from run to run in
- * both (the reference's sequence-parallel mode, _triton_kernels_v2.py:336-339, allows run-to-run
- * differences but does not require them).  The fp32 atomic-add formulation was measured on
- * MI355X and rejected: the L2 retires about 1.35 TB/s of fp32 atomic adds whatever their
- * locality, so the dQ contributions of a key-tile-parallel backward alone would take longer than
- * the whole two-kernel backward.
- * `workspace` is accepted for interface stability; fa2_bwd_workspace_bytes returns 0 and NULL is
- * fine.
+ * With FA2_CONFIG_AUTO both values of `deterministic` run the same two kernels: a key-tile-parallel
+ * kernel for dK and dV and a query-tile-parallel kernel that accumulates dQ in registers in a fixed
+ * order and writes it once.  There are no atomics, so results are bit-identical from run to run in
+ * both modes (the reference's sequence-parallel mode, _triton_kernels_v2.py:336-339, allows
+ * run-to-run differences but does not require them); fa2_bwd_workspace_bytes is 0 and `workspace`
+ * may be NULL.
+ * The reference's sequence-parallel formulation itself - one kernel per key tile that also adds its
+ * dQ contributions into an fp32 accumulator with global atomics (_triton_kernels_v2.py:336-339,
+ * 466-494), then dq = accumulator (flash_attention_2.py:277) - is the set of table rows with
+ * dq_atomic = 1, selected by passing their id as config_id with deterministic = 0 and a workspace
+ * of fa2_bwd_workspace_bytes() bytes.  It exists for head dimensions 32, 64 and 128 on 16-byte
+ * aligned tensors (FA2_ERR_BAD_CONFIG otherwise), needs dq, dk and dv together, and its dq may
+ * differ in the last bits from run to run.  The table never picks it: on MI355X the L2 retires
+ * about 1.35 TB/s of fp32 atomic adds whatever their locality, so it is 2-3 times slower than the
+ * two-kernel backward.
  * dK/dV and dQ are computed by two kernels launched back to back on `stream`.  A caller that
  * needs only part of the gradient (or wants to time one kernel) may pass dq == NULL to skip the
  * dQ kernel, or dk == dv == NULL to skip the dK/dV kernel; dk and dv are given or omitted

@@ -47,8 +47,9 @@ def test_abi_version_and_table(capi):
     lib = capi.load()
     assert lib.fa2_abi_version() == capi.ABI_VERSION
     rows = capi.config_table()
-    assert [r["headdim_padded"] for r in rows] == sorted(r["headdim_padded"] for r in rows)
-    assert rows[-1]["headdim_padded"] == capi.FA2_MAX_HEADDIM
+    auto = [r for r in rows if not r["dq_atomic"]]  # the rows the table picks from by itself
+    assert [r["headdim_padded"] for r in auto] == sorted(r["headdim_padded"] for r in auto)
+    assert auto[-1]["headdim_padded"] == capi.FA2_MAX_HEADDIM
     for r in rows:
         assert r["fwd_block_q"] == 32 * r["fwd_waves"]
         assert r["bwd_block_kv"] == 32 * r["bwd_waves"]
@@ -218,6 +219,25 @@ def test_noalloc_entry_point_refuses_sizes_beyond_its_scratch(capi):
     status = lib.fa2_bwd_fused_noalloc(*args)
     assert lib.fa2_status_string(status) == b"FA2_ERR_TOO_LARGE"
     assert b"FA2_NOALLOC_MAX_ROWS" in lib.fa2_last_error_string()
+
+
+def test_sequence_parallel_rows_and_workspace(capi, fa2_module):
+    """The table's sequence-parallel rows are never picked automatically, size their workspace, and
+    the configuration classes select them."""
+    lib = capi.load()
+    rows = capi.config_table()
+    atomic = [r for r in rows if r["dq_atomic"]]
+    assert sorted(r["headdim_padded"] for r in atomic) == [32, 64, 128]
+    for d in (8, 32, 64, 96, 128, 200, 256):
+        assert rows[lib.fa2_pick_config(capi.FA2_DTYPE_BF16, d, 512, 512, 0)]["dq_atomic"] == 0
+    for r in atomic:
+        d = r["headdim_padded"]
+        assert lib.fa2_bwd_workspace_bytes(2, 3, 130, 77, d, 0, r["id"]) == 2 * 3 * 192 * d * 4
+        assert lib.fa2_bwd_workspace_bytes(2, 3, 130, 77, d, 0, capi.FA2_CONFIG_AUTO) == 0
+    assert fa2_module.GFX950_KERNEL_CONFIG_SEQUENCE_PARALLEL_ATOMIC.atomic_dq
+    assert not fa2_module.GFX950_KERNEL_CONFIG_SEQUENCE_PARALLEL_ATOMIC.deterministic
+    assert not fa2_module.GFX950_KERNEL_CONFIG_NON_DETERMINISTIC.atomic_dq
+    assert not fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC.atomic_dq
 
 
 def test_workload_table_matches_baseline(workloads):
