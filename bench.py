@@ -234,6 +234,23 @@ def _kernel_legs(capi, w, q, k, v, d_o, iters: int):
         "bwd_dkdv": lambda: bwd(0, want_dq=False),
         "bwd_dq": lambda: bwd(0, want_dkdv=False),
     }
+    # The sequence-parallel backward run the reference's way (table rows with dq_atomic: one kernel
+    # per key tile, dQ accumulated with fp32 global atomics; never picked automatically): the whole
+    # call, i.e. accumulator clear + that kernel + conversion, preprocess not included, so that the
+    # figure compares with bwd_deterministic / bwd_sequence_parallel above.
+    atomic_rows = {r["headdim_padded"]: r["id"] for r in capi.config_table() if r["dq_atomic"]}
+    if d in atomic_rows:
+        row = atomic_rows[d]
+        ws_atomic = torch.empty(lib.fa2_bwd_workspace_bytes(b, h, n, n, d, 0, row), dtype=torch.uint8, device=q.device)
+
+        def bwd_atomic():
+            capi.check(lib.fa2_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), d_o.data_ptr(),
+                                   lse.data_ptr(), delta.data_ptr(), ws_atomic.data_ptr(),
+                                   dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                   b, h, n, n, d, n_r, *s3(q), *s3(k), *s3(v), *s3(d_o),
+                                   *s3(dq), *s3(dk), *s3(dv), scale, dtype, 0, row, stream), "fa2_bwd (dq_atomic row)")
+
+        legs["bwd_sequence_parallel_atomic"] = bwd_atomic
     for name, fn in legs.items():
         fn()
         torch.cuda.synchronize()
