@@ -55,12 +55,6 @@ struct Elem<__bf16> {
   static __device__ __forceinline__ float to_float(short x) {
     return __builtin_bit_cast(float, ((unsigned)(unsigned short)x) << 16);
   }
-  // acc + lo(pair) + hi(pair) for a packed pair of values (v_dot2c_f32_bf16 with a vector of ones).
-  static __device__ __forceinline__ float add_pair(unsigned pair, float acc) {
-    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair), ones, acc, false);
-  }
 };
 
 template <>
@@ -83,11 +77,6 @@ struct Elem<_Float16> {
   }
   static __device__ __forceinline__ float to_float(short x) {
     return (float)__builtin_bit_cast(_Float16, x);
-  }
-  static __device__ __forceinline__ float add_pair(unsigned pair, float acc) {
-    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pair), ones, acc, false);
   }
 };
 
