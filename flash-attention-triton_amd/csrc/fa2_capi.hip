@@ -37,14 +37,18 @@ using fa2::kDqBlockKV;
 using fa2::kDqBlockQ;
 using fa2::kFwdBlockKV;
 using fa2::kFwdBlockQ;
-constexpr int kHeadGroup = 64;  // (batch, head) pairs dispatched together: 8 per XCD
+// (batch, head) pairs dispatched together: 8 per XCD, or 4 at head dimension 128, where a head's K and
+// V rows are twice as large (C3, 64 heads: forward -0.9 %, dQ -1.3 % with 32 against 64; 16 costs
+// 2-4 %; at head dimension 64 a group of 32 costs 5-10 %).
+constexpr int kHeadGroup = 64;
+constexpr int kHeadGroup128 = 32;
 
 const fa2_config_info kTable[] = {
     // id DP  fwd:BQ       BKV        waves dK/dV:BQ   BKV       waves dQ:BQ    BKV      waves fast fwd/CU dq/CU dkdv/CU stages passes group
     {0, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 4, 3, 3, 1, kHeadGroup, 0},
     {1, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 3, 2, 3, 1, kHeadGroup, 0},
     {2, 96, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup, 0},
-    {3, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup, 0},
+    {3, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup128, 0},
     {4, 192, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 1, kHeadGroup, 0},
     {5, 256, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 2, kHeadGroup, 0},
     // Sequence-parallel rows (dq_atomic = 1): the backward is one key-tile-parallel kernel that adds its
@@ -54,18 +58,20 @@ const fa2_config_info kTable[] = {
     // a caller selects them by id.  Forward columns as in the row of the same head dimension.
     {6, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 0, 1, 3, 1, kHeadGroup, 1},
     {7, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 0, 1, 3, 1, kHeadGroup, 1},
-    {8, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 0, 1, 3, 1, kHeadGroup, 1},
+    {8, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 0, 1, 3, 1, kHeadGroup128, 1},
 };
 constexpr int kTableRows = sizeof(kTable) / sizeof(kTable[0]);
 
-// Heads dispatched together.  Up to twice the table's group size all heads form one group, so that
-// the whole grid is walked heaviest tile first: with 96 heads, a group of 64 followed by one of 32
-// starts the second group's heaviest tiles halfway through the kernel and they finish alone.
-// Beyond that the table's size applies (a multiple of 8: heads stay on one XCD).
+// Heads dispatched together by the forward and dQ kernels.  The heads are split into
+// floor(heads / group) groups of (nearly) equal size, each a multiple of 8 so that a head stays on
+// one XCD: equal groups, because a small last group would start its heaviest tiles late and finish
+// them alone (96 heads as 64 + 32 cost 5 % against one group of 96), and fewer than two table
+// groups' worth of heads form a single group, walked heaviest tile first over the whole grid.
 int head_group(int cfg, int64_t heads) {
   const int g = kTable[cfg].head_group;
-  if (heads <= 2 * g) return (int)((heads + 7) / 8 * 8);
-  return g;
+  const int64_t n_groups = heads / g > 0 ? heads / g : 1;
+  const int64_t per_group = (heads + n_groups - 1) / n_groups;
+  return (int)((per_group + 7) / 8 * 8);
 }
 
 int pick_config(int headdim) {
