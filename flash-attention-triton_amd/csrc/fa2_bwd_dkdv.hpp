@@ -535,7 +535,6 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 && !ATOMIC_DQ ? 2 : 1)) v
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- dP = dO V^T (ringb: dO rows -> Q^T); exponentials under the MFMAs -------------------
-    f32x16 pr;
     const int rel = qb + row_shift;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
@@ -556,16 +555,15 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 && !ATOMIC_DQ ? 2 : 1)) v
       for (int i = part(16, KS, ks); i < part(16, KS, ks + 1); i++) {
         float x = fast_exp2(s[i] * scale_log2 - l4[i >> 2][i & 3]);
         if (MASKED && (unsigned)(rel + (8 * (i >> 2) + (i & 3))) >= row_span) x = 0.f;
-        pr[i] = x;
+        s[i] = x;  // P takes the place of S
       }
-      asm volatile("" : "+v"(pr));
+      asm volatile("" : "+v"(s));
       __builtin_amdgcn_sched_barrier(0);
     }
-    f32x8 plo = {pr[0], pr[1], pr[2], pr[3], pr[4], pr[5], pr[6], pr[7]};
-    f32x8 phi = {pr[8], pr[9], pr[10], pr[11], pr[12], pr[13], pr[14], pr[15]};
+    f32x8 plo = {s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7]};
+    f32x8 phi = {s[8], s[9], s[10], s[11], s[12], s[13], s[14], s[15]};
     const s16x8 pf[2] = {Elem<T>::pack8(plo), Elem<T>::pack8(phi)};
     // ---- dV^T += dO^T P (ring: dO^T -> Q rows of the next block); dS arithmetic under the MFMAs
-    f32x16 ds;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       dvacc[ks % DB] = Elem<T>::mfma(ring[ks], pf[ks / DB], dvacc[ks % DB]);
@@ -573,12 +571,12 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 && !ATOMIC_DQ ? 2 : 1)) v
       ring[ks] = lds_read_128(qnext[ks] + (HALF == 0 ? 32 * LP : 0));
       if (ks == 0) settle(dp);
 #pragma unroll
-      for (int i = part(16, KS, ks); i < part(16, KS, ks + 1); i++) ds[i] = pr[i] * dp[i];
-      asm volatile("" : "+v"(ds));
+      for (int i = part(16, KS, ks); i < part(16, KS, ks + 1); i++) dp[i] = s[i] * dp[i];  // dS takes the place of dP
+      asm volatile("" : "+v"(dp));
       __builtin_amdgcn_sched_barrier(0);
     }
-    f32x8 dlo = {ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]};
-    f32x8 dhi = {ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]};
+    f32x8 dlo = {dp[0], dp[1], dp[2], dp[3], dp[4], dp[5], dp[6], dp[7]};
+    f32x8 dhi = {dp[8], dp[9], dp[10], dp[11], dp[12], dp[13], dp[14], dp[15]};
     const s16x8 dsf[2] = {Elem<T>::pack8(dlo), Elem<T>::pack8(dhi)};
     if (ATOMIC_DQ) {
       // This lane's key row of dS: element j of dsf[t] is query 16 t + 8 (j / 4) + 4 h + j % 4.
