@@ -49,8 +49,8 @@ const fa2_config_info kTable[] = {
     {1, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 3, 2, 3, 1, kHeadGroup, 0},
     {2, 96, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup, 0},
     {3, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup128, 0},
-    {4, 192, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 1, kHeadGroup, 0},
-    {5, 256, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 0, 1, 1, 1, 2, 2, kHeadGroup, 0},
+    {4, 192, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 2, 1, 1, 1, 2, 1, kHeadGroup, 0},
+    {5, 256, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 2, 1, 1, 1, 2, 2, kHeadGroup, 0},
     // Sequence-parallel rows (dq_atomic = 1): the backward is one key-tile-parallel kernel that adds its
     // dQ contributions into an fp32 workspace with global atomics, the reference's non-deterministic
     // formulation (_triton_kernels_v2.py:336-339).  Never picked automatically: on MI355X the atomics

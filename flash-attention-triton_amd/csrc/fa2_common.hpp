@@ -243,6 +243,10 @@ template <int DP>
 __device__ __forceinline__ int swz(int r);
 template <>
 __device__ __forceinline__ int swz<128>(int r) { return 4 * (r & 3) + ((r >> 2) & 3); }
+// Rows of 256 halves span the 64 banks twice: the bank of a slot is its low four bits, so the
+// 128-column pattern applied to those bits keeps both access patterns conflict-free.
+template <>
+__device__ __forceinline__ int swz<256>(int r) { return swz<128>(r); }
 template <>
 __device__ __forceinline__ int swz<64>(int r) { return 4 * ((r >> 1) & 1) + ((r >> 2) & 3); }
 template <>
@@ -304,7 +308,7 @@ __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0
 // Row pitch, in elements, of the LDS tiles of the fast kernels for head dimension DP.  The swizzle
 // needs a power-of-two number of 16-byte chunks per row, so 96 columns live in rows of 128: the
 // last four chunk slots of a row are never loaded and never read.
-constexpr int lds_pitch(int dp) { return dp == 96 ? 128 : dp; }
+constexpr int lds_pitch(int dp) { return dp == 96 ? 128 : dp == 192 ? 256 : dp; }
 
 // Items [part(n, units, u), part(n, units, u + 1)) are unit u's share of n items spread as evenly
 // as integers allow over `units` units (equal shares when units divides n).
@@ -340,8 +344,11 @@ struct TileLoader {
   static constexpr int LOADS = NL / NW; // per wave
   static_assert(NL % NW == 0 && LOADS >= 1, "tile must split evenly over the waves");
   // Multiples of NW*RPL rows keep the low four row bits the swizzle looks at, so a lane's
-  // swizzled chunk does not depend on the load index.
-  static_assert((NW * RPL) % 16 == 0, "swizzle must be independent of the load index");
+  // swizzled chunk does not depend on the load index.  Rows of 256 halves (two rows per wave-load,
+  // eight rows per round of the four waves) are the exception: row bit 3 alternates with the load
+  // index and flips bit 1 of the swizzle, so a lane has one chunk for even loads and one for odd.
+  static constexpr bool BY_PARITY = (NW * RPL) % 16 != 0;
+  static_assert(!BY_PARITY || (NW * RPL == 8 && LP == 256), "swizzle must be independent of the load index");
   static constexpr int TILE_ELEMS = ROWS * LP;
 
   const short *base;  // first row of the matrix for this (batch, head)
@@ -351,6 +358,9 @@ struct TileLoader {
   int chunk;          // this lane's global chunk index
   unsigned voff;      // byte offset of this lane inside a tile for load 0
   bool active;        // this lane's slot holds data
+  int chunk_odd;      // BY_PARITY: the same three for odd load indices
+  unsigned voff_odd;
+  bool active_odd;
 
   static constexpr bool ALL_ACTIVE = LP == DP && !PAD;  // every slot of a row holds data
 
@@ -362,6 +372,9 @@ struct TileLoader {
     chunk = (lane % CPR) ^ swz<LP>(row_in);
     active = ALL_ACTIVE || chunk < (PAD ? chunks : DP / 8);
     voff = 2u * (unsigned)(row_in * (int)stride + chunk * 8);
+    chunk_odd = BY_PARITY ? chunk ^ 2 : chunk;
+    active_odd = ALL_ACTIVE || chunk_odd < (PAD ? chunks : DP / 8);
+    voff_odd = 2u * (unsigned)(row_in * (int)stride + chunk_odd * 8);
   }
 
   // Rows [row0, row0 + ROWS), all inside the matrix -> tile at LDS byte address `lds`.
@@ -374,8 +387,10 @@ struct TileLoader {
   // between other work.
   __device__ __forceinline__ void issue_one(int row0, unsigned lds, int i) const {
     const short *tile = base + (int64_t)row0 * stride;
-    if (ALL_ACTIVE || active)
-      load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, voff, lds + (unsigned)(i * NW + wave) * 1024u);
+    const bool odd = BY_PARITY && (i & 1);
+    if (ALL_ACTIVE || (odd ? active_odd : active))
+      load_lds_16(tile + (int64_t)(i * NW * RPL) * stride, odd ? voff_odd : voff,
+                  lds + (unsigned)(i * NW + wave) * 1024u);
   }
 
   // Same, but rows at or beyond `nrows` are taken from row nrows - 1 (finite values that the
@@ -384,8 +399,10 @@ struct TileLoader {
 #pragma unroll
     for (int i = 0; i < LOADS; i++) {
       const int r = min(row0 + i * NW * RPL + row_in, nrows - 1);
-      if (ALL_ACTIVE || active)
-        load_lds_16(base + (int64_t)r * stride + chunk * 8, lds + (unsigned)(i * NW + wave) * 1024u);
+      const bool odd = BY_PARITY && (i & 1);
+      if (ALL_ACTIVE || (odd ? active_odd : active))
+        load_lds_16(base + (int64_t)r * stride + (odd ? chunk_odd : chunk) * 8,
+                    lds + (unsigned)(i * NW + wave) * 1024u);
     }
   }
 };

@@ -252,7 +252,10 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_kerne
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast path: head dimension equal to the padded one and 16-byte aligned rows.
+// Fast path: 16-byte aligned rows and a head dimension that is a multiple of 8; instantiated for 32,
+// 64, 96, 128, 192 and 256 columns (two workgroups or more per CU up to 128; at 192 and 256 the
+// five tile stages fill the CU's 160 KiB of LDS and the output accumulator moves into accumulation
+// registers: one workgroup per CU, one wave per SIMD).
 //
 //  * K and V tiles (64 rows) go straight from global memory into swizzled, unpadded LDS
 //    (global_load_lds_dwordx4: no staging registers, no LDS stores); three K stages and two V
@@ -293,7 +296,7 @@ struct HalfTag {
 // PAD: the head dimension is a multiple of 8 below DP; the columns beyond it are zeros in LDS and in
 // the register fragments, and are not stored.
 template <typename T, int DP, int BKV, bool PAD>
-__global__ __launch_bounds__(64 * kFwdWaves, 2) void fwd_direct_kernel(const FwdParams p) {
+__global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direct_kernel(const FwdParams p) {
   using L = FwdDirectLayout<DP, BKV>;
   constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
   constexpr int NTHREADS = 64 * kFwdWaves;

@@ -23,7 +23,9 @@ void launch_direct(int dp, const FwdParams &p, dim3 grid, dim3 block, hipStream_
     case 32: hipLaunchKernelGGL((fwd_direct_kernel<T, 32, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
     case 64: hipLaunchKernelGGL((fwd_direct_kernel<T, 64, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
     case 96: hipLaunchKernelGGL((fwd_direct_kernel<T, 96, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fwd_direct_kernel<T, 128, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
+    case 128: hipLaunchKernelGGL((fwd_direct_kernel<T, 128, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
+    case 192: hipLaunchKernelGGL((fwd_direct_kernel<T, 192, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fwd_direct_kernel<T, 256, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
   }
 }
 

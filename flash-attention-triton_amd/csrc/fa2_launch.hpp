@@ -12,15 +12,19 @@ namespace fa2 {
 // Which kernel a launcher picked (reported to callers that label measurements).
 enum KernelPath { kPathGeneric = 0, kPathDirect = 1 };
 
-// The fast kernels need a head dimension that is a multiple of 8 (whole 16-byte chunks) up to 128,
+// The fast kernels need a head dimension that is a multiple of 8 (whole 16-byte chunks) up to 128
+// (up to 256 in the forward),
 // 16-byte aligned rows and row offsets inside a tile that fit 32 bits.  A head dimension below the
 // table row's padded one runs the padded variant of the kernel.
 inline bool direct_stride_ok(const Tensor4 &t) { return t.stride_seq < (int64_t(1) << 24); }
 inline bool direct_headdim(int dp, int headdim) {
   return headdim % 8 == 0 && headdim <= dp && (dp == 32 || dp == 64 || dp == 96 || dp == 128);
 }
+// The forward also has fast kernels for the rows of 192 and 256 columns (one wave per SIMD, all
+// 160 KiB of LDS).
 inline bool fwd_direct_ok(int dp, const FwdParams &p) {
-  return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
+  const bool hd = direct_headdim(dp, p.headdim) || (p.headdim % 8 == 0 && p.headdim <= dp && (dp == 192 || dp == 256));
+  return p.vec && hd && direct_stride_ok(p.k) && direct_stride_ok(p.v);
 }
 inline bool dq_direct_ok(int dp, const BwdParams &p) {
   return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);

@@ -79,6 +79,12 @@ SMALL_CASES = [
     (1, 2, 333, 200, 192, torch.float16, 1.0),
     (2, 2, 300, 300, 256, torch.bfloat16, 1.0),
     (1, 1, 130, 130, 250, torch.float16, 1.0),    # above 128 and not a multiple of 8
+    # several tiles at head dims above 128 (LDS-direct forward with rows of 256 in LDS, generic backward)
+    (1, 2, 450, 200, 256, torch.bfloat16, 1.0),
+    (1, 2, 200, 450, 192, torch.float16, 1.0),
+    (2, 1, 333, 333, 200, torch.bfloat16, 1.0),   # padded into the row of 256
+    (1, 2, 700, 700, 248, torch.float16, 1.0),
+    (1, 1, 600, 600, 136, torch.float16, 3.0),    # padded into the row of 192, peaky softmax
     # head dims that are a multiple of 8 below the table row's: the padded LDS-direct kernels
     (2, 2, 333, 333, 8, torch.float16, 1.0),
     (1, 2, 200, 450, 24, torch.bfloat16, 1.0),
@@ -112,6 +118,26 @@ def test_golden_fixtures(fa, fa2_module, name):
 
 
 # ------------------------------------------------------------------------- lse and delta through the launchers / C ABI
+@pytest.mark.parametrize("shape", [(1, 2, 450, 300, 256, torch.bfloat16), (2, 1, 333, 500, 192, torch.float16),
+                                   (1, 2, 513, 513, 160, torch.bfloat16)],
+                         ids=lambda c: f"Nq{c[2]}Nk{c[3]}D{c[4]}")
+def test_lse_at_large_head_dims(fa2_module, shape):
+    """The forward kernels for head dimensions above 128 write the same lse layout (per-head check
+    against logsumexp of the masked scores)."""
+    b, h, nq, nk, d, dtype = shape
+    q, k, v, _ = _seeded((b, h, nq, d), (b, h, nk, d), dtype)
+    cfg = fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC
+    scale = 1 / math.sqrt(d)
+    out, lse, _ = fa2_module._flash_attention_forward(
+        q.cuda(), k.cuda(), v.cuda(), scale, cfg.block_rows_size, cfg.block_cols_size, cfg.min_block_headdim,
+        cfg.max_headdim, cfg.seqlen_cache_divisor, cfg.min_warps, cfg.max_warps, cfg.num_stages)
+    torch.cuda.synchronize()
+    want = oracle.naive_lse(q, k, scale)
+    _assert_close("lse", lse[..., :nq], want, atol=2e-3, rtol=1e-3)
+    assert torch.count_nonzero(lse[..., nq:]) == 0, "padded lse rows must be written as zero"
+    _assert_close("o", out, oracle.naive_causal_attention(q, k, v, scale))
+
+
 @pytest.mark.parametrize("name", golden_io.NAMES)
 def test_lse_and_delta_match_oracle(fa2_module, capi, name):
     g = golden_io.load(name)
