@@ -269,7 +269,7 @@ struct DqDirectLayout {
 // PAD: the head dimension is a multiple of 8 below DP; the columns beyond it are zeros in LDS and in
 // the register fragments, and are not stored.
 template <typename T, int DP, int BKV, bool FUSE_DELTA, bool PAD>
-__global__ __launch_bounds__(64 * kDqWaves, 2) void bwd_dq_direct_kernel(const BwdParams p) {
+__global__ __launch_bounds__(64 * kDqWaves, (DP <= 128 ? 2 : 1)) void bwd_dq_direct_kernel(const BwdParams p) {
   using L = DqDirectLayout<DP, BKV>;
   constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
   constexpr int BLK = 32;

@@ -11,7 +11,9 @@ void launch_direct_pad(int dp, const BwdParams &p, dim3 grid, dim3 block, hipStr
     case 32: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 32, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
     case 64: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 64, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
     case 96: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 96, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 128, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
+    case 128: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 128, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
+    case 192: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 192, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((bwd_dq_direct_kernel<T, 256, kDqBlockKV, FUSE_DELTA, PAD>), grid, block, 0, s, p); break;
   }
 }
 

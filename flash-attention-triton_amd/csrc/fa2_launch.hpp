@@ -20,14 +20,16 @@ inline bool direct_stride_ok(const Tensor4 &t) { return t.stride_seq < (int64_t(
 inline bool direct_headdim(int dp, int headdim) {
   return headdim % 8 == 0 && headdim <= dp && (dp == 32 || dp == 64 || dp == 96 || dp == 128);
 }
-// The forward also has fast kernels for the rows of 192 and 256 columns (one wave per SIMD, all
-// 160 KiB of LDS).
+// The forward and dQ kernels, which stream K and V, also have fast variants for the rows of 192 and
+// 256 columns (one wave per SIMD, all 160 KiB of LDS).
+inline bool direct_headdim_kv_stream(int dp, int headdim) {
+  return direct_headdim(dp, headdim) || (headdim % 8 == 0 && headdim <= dp && (dp == 192 || dp == 256));
+}
 inline bool fwd_direct_ok(int dp, const FwdParams &p) {
-  const bool hd = direct_headdim(dp, p.headdim) || (p.headdim % 8 == 0 && p.headdim <= dp && (dp == 192 || dp == 256));
-  return p.vec && hd && direct_stride_ok(p.k) && direct_stride_ok(p.v);
+  return p.vec && direct_headdim_kv_stream(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
 }
 inline bool dq_direct_ok(int dp, const BwdParams &p) {
-  return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
+  return p.vec && direct_headdim_kv_stream(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
 }
 inline bool dkdv_direct_ok(int dp, const BwdParams &p) {
   return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.q) && direct_stride_ok(p.d_o);
