@@ -79,7 +79,7 @@ typedef struct fa2_config_info {
   int dq_block_kv;
   int dq_waves;
   int lds_direct;     /* the row's LDS-direct kernels (global_load_lds into swizzled tiles): 0 none, 1 forward and
-                         backward, 2 forward only (one wave per SIMD, all 160 KiB of LDS; generic backward) */
+                         backward, 2 forward and dQ only (one wave per SIMD, all 160 KiB of LDS; generic dK/dV) */
   int fwd_wg_per_cu;  /* workgroups that share a CU (what registers and LDS leave room for) */
   int dq_wg_per_cu;
   int dkdv_wg_per_cu;
