@@ -58,6 +58,11 @@ def test_abi_version_and_table(capi):
                     (129, 192), (192, 192), (193, 256), (256, 256)):
         idx = lib.fa2_pick_config(capi.FA2_DTYPE_BF16, d, 512, 512, 0)
         assert idx >= 0 and rows[idx]["headdim_padded"] == want
+    # LDS-direct kernels: all three up to 128 columns, forward and dQ only at 192 and 256.
+    assert [r["lds_direct"] for r in auto] == [1, 1, 1, 1, 2, 2]
+    # (batch, head) pairs dispatched together: a multiple of 8 (one XCD per head), fewer at 128 columns.
+    assert all(r["head_group"] % 8 == 0 and r["head_group"] > 0 for r in rows)
+    assert {r["headdim_padded"]: r["head_group"] for r in auto}[128] < {r["headdim_padded"]: r["head_group"] for r in auto}[64]
     assert lib.fa2_pick_config(capi.FA2_DTYPE_BF16, 257, 512, 512, 0) == -4  # FA2_ERR_HEADDIM
     assert lib.fa2_pick_config(7, 64, 512, 512, 0) == -3  # FA2_ERR_BAD_DTYPE
     info = capi.ConfigInfo()
