@@ -264,9 +264,10 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_kerne
 //    vector work of the same wave next to it (about four VALU instructions issue for free under
 //    a 32x32x16 MFMA, and short alternating phases are also what lets two waves of one SIMD
 //    overlap).  For block j:
-//        X(j): S_{j+1}^T = K_{j+1} Q^T   interleaved with   P_j = exp2(scale*S_j - m), row sums
-//        Y(j): O^T += V_j^T P_j^T         interleaved with   row maximum of S_{j+1}
-//    The two score buffers alternate roles, so pipelining costs no extra registers.
+//        X(j): S_{j+1}^T = K_{j+1} Q^T   interleaved with   packing P_j for the MFMA
+//        Y(j): O^T += V_j^T P_j^T         interleaved with   P_{j+1} = exp2(scale*S_{j+1} - m), row sums
+//    One score buffer and one probability buffer are enough: each is consumed in the phase after
+//    the one that fills it.
 //  * MFMA operand fragments travel through a ring of DP/16 register sets that is refilled as it
 //    is consumed (K fragments of block j+2 during Y(j), V fragments of block j during X(j)), so
 //    LDS latency hides behind the MFMAs.
@@ -447,8 +448,8 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
 
   // One block step.  On entry e holds the probabilities of block j (formed against m_ref) and the
   // ring the K fragments of block j+1.
-  //     X: S_{j+1}^T = K_{j+1} Q^T   beside   pack P_j, add its row sums        ring <- V_j^T
-  //     Y: O^T += V_j^T P_j^T        beside   max and exponentials of S_{j+1}   ring <- K_{j+2}
+  //     X: S_{j+1}^T = K_{j+1} Q^T   beside   pack P_j                                  ring <- V_j^T
+  //     Y: O^T += V_j^T P_j^T        beside   exponentials of S_{j+1} and their row sums   ring <- K_{j+2}
   // The exponentials, which do not overlap with MFMAs of their own wave and are the most expensive
   // vector instructions here, sit in the phase whose MFMAs need the fewest LDS reads, which evens
   // out the two phases.  HALF (= j & 1) selects the half-tile: V_j is half HALF of the current V
