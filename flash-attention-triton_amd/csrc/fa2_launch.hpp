@@ -13,9 +13,9 @@ namespace fa2 {
 enum KernelPath { kPathGeneric = 0, kPathDirect = 1 };
 
 // The fast kernels need a head dimension that is a multiple of 8 (whole 16-byte chunks) up to 128
-// (up to 256 in the forward),
-// 16-byte aligned rows and row offsets inside a tile that fit 32 bits.  A head dimension below the
-// table row's padded one runs the padded variant of the kernel.
+// (up to 256 in the forward and dQ kernels), 16-byte aligned rows and row offsets inside a tile that
+// fit 32 bits.  A head dimension below the table row's padded one runs the padded variant of the
+// kernel.
 inline bool direct_stride_ok(const Tensor4 &t) { return t.stride_seq < (int64_t(1) << 24); }
 inline bool direct_headdim(int dp, int headdim) {
   return headdim % 8 == 0 && headdim <= dp && (dp == 32 || dp == 64 || dp == 96 || dp == 128);
