@@ -240,21 +240,21 @@ __device__ __forceinline__ void map_workgroup(int i, int heads, int tiles_per_he
 // (slot s of row r is loaded from chunk s ^ swz(r)).
 // ------------------------------------------------------------------------------------------
 template <int DP>
-__device__ __forceinline__ int swz(int r);
+__host__ __device__ __forceinline__ int swz(int r);
 template <>
-__device__ __forceinline__ int swz<128>(int r) { return 4 * (r & 3) + ((r >> 2) & 3); }
+__host__ __device__ __forceinline__ int swz<128>(int r) { return 4 * (r & 3) + ((r >> 2) & 3); }
 // Rows of 256 halves span the 64 banks twice: the bank of a slot is its low four bits, so the
 // 128-column pattern applied to those bits keeps both access patterns conflict-free.
 template <>
-__device__ __forceinline__ int swz<256>(int r) { return swz<128>(r); }
+__host__ __device__ __forceinline__ int swz<256>(int r) { return swz<128>(r); }
 template <>
-__device__ __forceinline__ int swz<64>(int r) { return 4 * ((r >> 1) & 1) + ((r >> 2) & 3); }
+__host__ __device__ __forceinline__ int swz<64>(int r) { return 4 * ((r >> 1) & 1) + ((r >> 2) & 3); }
 template <>
-__device__ __forceinline__ int swz<32>(int r) { return (r >> 2) & 3; }
+__host__ __device__ __forceinline__ int swz<32>(int r) { return (r >> 2) & 3; }
 
 // Element offset of (row r, logical chunk c) in a swizzled tile.
 template <int DP>
-__device__ __forceinline__ int swz_off(int r, int c) { return r * DP + ((c ^ swz<DP>(r)) << 3); }
+__host__ __device__ __forceinline__ int swz_off(int r, int c) { return r * DP + ((c ^ swz<DP>(r)) << 3); }
 
 // LDS-direct load of 16 bytes per lane: lane l's data lands at lds_wave_base + 16*l.
 // Written as inline assembly on purpose: with the compiler builtin every later LDS read is made
@@ -364,15 +364,23 @@ struct TileLoader {
 
   static constexpr bool ALL_ACTIVE = LP == DP && !PAD;  // every slot of a row holds data
 
+  // Wave-load i of wave `wave` fills LDS bytes [(i * NW + wave) * 1024, + 1024) of the tile, lane l
+  // the 16 bytes at 16 * l: slot l % CPR of tile row i * NW * RPL + wave * RPL + l / CPR.  This is the
+  // global 16-byte chunk of that row which the slot holds under the swizzle.
+  static __host__ __device__ __forceinline__ int chunk_of(int lane, int wave, int i) {
+    const int row = i * NW * RPL + wave * RPL + lane / CPR;
+    return (lane % CPR) ^ swz<LP>(row);
+  }
+
   __device__ __forceinline__ TileLoader(const short *base_, int64_t stride_, int chunks = DP / 8)
       : base(base_), stride(stride_) {
     const int lane = threadIdx.x & 63;
     wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     row_in = wave * RPL + lane / CPR;
-    chunk = (lane % CPR) ^ swz<LP>(row_in);
+    chunk = (lane % CPR) ^ swz<LP>(row_in);  // == chunk_of(lane, wave, 0)
     active = ALL_ACTIVE || chunk < (PAD ? chunks : DP / 8);
     voff = 2u * (unsigned)(row_in * (int)stride + chunk * 8);
-    chunk_odd = BY_PARITY ? chunk ^ 2 : chunk;
+    chunk_odd = BY_PARITY ? chunk ^ 2 : chunk;  // == chunk_of(lane, wave, odd i), see BY_PARITY
     active_odd = ALL_ACTIVE || chunk_odd < (PAD ? chunks : DP / 8);
     voff_odd = 2u * (unsigned)(row_in * (int)stride + chunk_odd * 8);
   }
