@@ -62,17 +62,9 @@ const fa2_config_info kTable[] = {
 };
 constexpr int kTableRows = sizeof(kTable) / sizeof(kTable[0]);
 
-// Heads dispatched together by the forward and dQ kernels.  The heads are split into
-// floor(heads / group) groups of (nearly) equal size, each a multiple of 8 so that a head stays on
-// one XCD: equal groups, because a small last group would start its heaviest tiles late and finish
-// them alone (96 heads as 64 + 32 cost 5 % against one group of 96), and fewer than two table
-// groups' worth of heads form a single group, walked heaviest tile first over the whole grid.
-int head_group(int cfg, int64_t heads) {
-  const int g = kTable[cfg].head_group;
-  const int64_t n_groups = heads / g > 0 ? heads / g : 1;
-  const int64_t per_group = (heads + n_groups - 1) / n_groups;
-  return (int)((per_group + 7) / 8 * 8);
-}
+// Heads dispatched together by the forward and dQ kernels: the table's group size, evened out over
+// the heads there are (fa2::equal_head_groups).
+int head_group(int cfg, int64_t heads) { return fa2::equal_head_groups(kTable[cfg].head_group, heads); }
 
 int pick_config(int headdim) {
   for (int i = 0; i < kTableRows; i++)

@@ -214,7 +214,7 @@ __device__ __forceinline__ void store_transposed_acc(const f32x16 (&acc)[DP / 32
 // Workgroups go to the 8 XCDs round-robin and `group` is a multiple of 8, so a head also stays on
 // one XCD (one L2), `group / 8` heads sharing that L2 at a time.  The group size comes from the
 // gfx950 table (per kernel and problem size).
-__device__ __forceinline__ void map_workgroup(int i, int heads, int tiles_per_head, int group, int &bh,
+__host__ __device__ __forceinline__ void map_workgroup(int i, int heads, int tiles_per_head, int group, int &bh,
                                               int &rank) {
   const int per_group = group * tiles_per_head;
   const int g = i / per_group;

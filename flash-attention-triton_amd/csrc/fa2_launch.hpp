@@ -40,6 +40,18 @@ inline bool seqpar_atomic_ok(int dp, const BwdParams &p) {
   return dkdv_direct_ok(dp, p) && p.headdim == dp && (dp == 32 || dp == 64 || dp == 128);
 }
 
+// Size of the head groups map_workgroup is given, for `heads` (batch, head) pairs and a table group
+// size `group`: the heads are split into floor(heads / group) groups of (nearly) equal size, each a
+// multiple of 8 so that a head stays on one XCD.  Equal groups, because a small last group would start
+// its heaviest tiles late and finish them alone (96 heads as 64 + 32 cost 5 % against one group of 96);
+// fewer than two table groups' worth of heads form a single group, walked heaviest tile first over
+// the whole grid.
+inline int equal_head_groups(int group, int64_t heads) {
+  const int64_t n_groups = heads / group > 0 ? heads / group : 1;
+  const int64_t per_group = (heads + n_groups - 1) / n_groups;
+  return (int)((per_group + 7) / 8 * 8);
+}
+
 // bf16 != 0 selects the bf16 kernels, otherwise fp16.
 void launch_fwd(bool bf16, int dp, const FwdParams &p, dim3 grid, hipStream_t s);
 void launch_preprocess(bool bf16, const PreParams &p, dim3 grid, hipStream_t s);

@@ -1,6 +1,7 @@
-// Host-side check of the LDS tile layout the fast kernels share (compiled for the host only and run
-// on the CPU by tests/test_lds_layout.py).  For every padded head dimension it walks all lanes, waves
-// and wave-loads of a 64-row tile and verifies that
+// Host-side check of index arithmetic the kernels and launchers share (compiled for the host only and
+// run on the CPU by tests/test_lds_layout.py): the workgroup -> (head, tile) mapping with its head
+// groups, and the LDS tile layout.  For every padded head dimension it walks all lanes, waves and
+// wave-loads of a 64-row tile and verifies that
 //   * the slot an LDS-direct load writes is where the fragment readers (swz_off) look for the chunk
 //     the loader fetched into it, and every (row, chunk) of the tile is written exactly once;
 //   * the loader's shortcut holds: the chunk does not depend on the load index, except with rows of
@@ -12,6 +13,7 @@
 #include <vector>
 
 #include "fa2_common.hpp"
+#include "fa2_launch.hpp"
 
 template <int DP>
 int check() {
@@ -57,8 +59,44 @@ int check() {
   return bad;
 }
 
+// Workgroup index -> (head, tile rank) with the head groups the launchers compute: every pair is
+// visited exactly once, ranks never decrease inside a group (heaviest tile first), group sizes are
+// multiples of 8, and with a head count that is a multiple of 8 all workgroups of a head have the
+// same index modulo 8, that is, land on one XCD.
+int check_mapping() {
+  int bad = 0, cases = 0;
+  for (int table_group : {32, 64})
+    for (int heads : {1, 3, 8, 16, 24, 33, 48, 63, 64, 72, 80, 96, 100, 128, 129, 192, 2048})
+      for (int tiles : {1, 2, 7, 32}) {
+        const int group = fa2::equal_head_groups(table_group, heads);
+        if (group % 8 != 0 || group < 8) bad++;
+        if (heads >= 2 * table_group && group > 2 * table_group) bad++;  // groups stay near the table's size
+        std::vector<int> seen(heads * tiles, 0), xcd(heads, -1);
+        int last_rank = 0, last_group = -1;
+        for (int i = 0; i < heads * tiles; i++) {
+          int bh = -1, rank = -1;
+          fa2::map_workgroup(i, heads, tiles, group, bh, rank);
+          if (bh < 0 || bh >= heads || rank < 0 || rank >= tiles) { bad++; continue; }
+          seen[bh * tiles + rank]++;
+          const int g = bh / group;
+          if (g == last_group && rank < last_rank) bad++;
+          if (g < last_group) bad++;  // groups are walked in order
+          last_group = g;
+          last_rank = rank;
+          if (heads % 8 == 0) {
+            if (xcd[bh] < 0) xcd[bh] = i % 8;
+            else if (xcd[bh] != i % 8) bad++;
+          }
+        }
+        for (int v : seen) bad += v != 1;
+        cases++;
+      }
+  printf("workgroup mapping, %d cases: %s\n", cases, bad ? "FAILED" : "ok");
+  return bad;
+}
+
 int main() {
-  int bad = 0;
+  int bad = check_mapping();
   bad += check<32>();
   bad += check<64>();
   bad += check<96>();

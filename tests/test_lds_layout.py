@@ -1,7 +1,7 @@
-"""The LDS tile layout of the fast kernels, checked on the CPU: tests/lds_layout_check.hip includes the
-kernels' own header (its swizzle and the tile loader's slot-to-chunk function are host-callable),
-is compiled for the host only and walks every lane, wave and wave-load of a tile for each padded
-head dimension."""
+"""Index arithmetic of the fast kernels, checked on the CPU: tests/lds_layout_check.hip includes the
+kernels' own headers (the swizzle, the tile loader's slot-to-chunk function, the workgroup mapping and the
+head-group rule are host-callable), is compiled for the host only, walks every lane, wave and wave-load
+of a tile for each padded head dimension and every workgroup of a range of grids."""
 
 from __future__ import annotations
 
@@ -28,3 +28,5 @@ def test_loader_slots_match_fragment_reads_and_reads_are_conflict_free(tmp_path)
     assert run.returncode == 0, run.stdout + run.stderr
     lines = [l for l in run.stdout.splitlines() if l.startswith("DP")]
     assert len(lines) == 6 and all(l.endswith("ok") for l in lines), run.stdout
+    mapping = [l for l in run.stdout.splitlines() if l.startswith("workgroup mapping")]
+    assert len(mapping) == 1 and mapping[0].endswith("ok"), run.stdout
