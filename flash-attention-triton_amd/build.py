@@ -44,11 +44,6 @@ def build(force: bool = True) -> pathlib.Path:
         raise RuntimeError(f"build did not produce {LIBRARY}")
     if force or not TORCH_EXTENSION.exists():
         build_torch_extension()
-    # The measurement probes next to the kernels (stand-alone executables under probes/bin).
-    cmd = ["make", "-j2", "-C", str(CSRC / "probes")]
-    if force:
-        cmd.append("-B")
-    subprocess.run(cmd, check=True)
     return LIBRARY
 
 

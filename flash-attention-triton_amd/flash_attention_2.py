@@ -216,7 +216,8 @@ def _flash_attention_backward(
     # (asserted above), so shapes, dtype, scale, mode and table row identify the record; the
     # workspace size is asked once per record (0 unless a sequence-parallel row was asked for: dQ
     # is written directly).
-    key = (q.shape, seqlen_k, q.dtype, softmax_scale, deterministic, config_id, threading.get_ident())
+    key = (q.shape, seqlen_k, q.dtype, seqlen_q_rounded, softmax_scale, deterministic, config_id,
+           threading.get_ident())
     cached = _BWD_ARGS.get(key)
     if cached is None:
         args = _capi.BwdArgs()
@@ -233,6 +234,8 @@ def _flash_attention_backward(
         cached = (args, ws_bytes)
         _remember(_BWD_ARGS, key, cached)
     args, ws_bytes = cached
+    # lse and delta rows are indexed with the record's row length: it must be the one they were allocated with.
+    assert lse.shape[2] == delta.shape[2] == args.seqlen_q_rounded
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     args.q.ptr, args.k.ptr, args.v.ptr = q.data_ptr(), k.data_ptr(), v.data_ptr()
     args.o.ptr, args.d_o.ptr = output.data_ptr(), d_output.data_ptr()

@@ -204,6 +204,36 @@ def test_launcher_assertions_mirror_reference(fa2_module):
         fwd(q, q, q, None, *tail)
 
 
+def test_backward_record_follows_the_lse_row_length(fa2_module, monkeypatch):
+    """The cached argument record of the backward launcher is per padded lse row length: the same
+    shapes under another max_headdim (N = 100 pads to 256 or to 128, flash_attention_2.py:98) must
+    not be handed the earlier call's seqlen_q_rounded, which the kernels index lse and delta with."""
+    seen = []
+
+    class FakeLibrary:
+        @staticmethod
+        def fa2_bwd_workspace_bytes(*_):
+            return 0
+
+        @staticmethod
+        def fa2_bwd_packed(args, _stream):
+            seen.append((args.seqlen_q, args.seqlen_q_rounded))
+            return 0
+
+    monkeypatch.setattr(fa2_module._capi, "load", lambda: FakeLibrary)
+    monkeypatch.setattr(fa2_module, "_stream_handle", lambda: 0)
+    base = fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC
+    q = torch.zeros(1, 2, 100, 64, dtype=torch.float16)
+    grads = [torch.empty_like(q) for _ in range(3)]
+    for max_headdim, rounded in ((256, 256), (128, 128), (256, 256)):
+        cfg = dataclasses.replace(base, max_headdim=max_headdim)
+        lse = torch.zeros(1, 2, rounded)
+        fa2_module._flash_attention_backward(q, q, q, q, lse, *grads, q, None, cfg)
+        with pytest.raises(AssertionError):  # an lse of another row length is refused, as in the reference
+            fa2_module._flash_attention_backward(q, q, q, q, torch.zeros(1, 2, rounded + 128), *grads, q, None, cfg)
+    assert seen == [(100, 256), (100, 128), (100, 256)]
+
+
 def test_cpp_autograd_node_is_built_and_matches_the_library(capi, fa2_module):
     """The C++ autograd node (csrc/fa2_torch_autograd.cpp) loads without a GPU, is linked against
     the same ABI as the ctypes binding, and is what the public functions record."""

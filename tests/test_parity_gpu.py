@@ -306,7 +306,7 @@ def test_constant_values_give_constant_output(fa, workloads):
 
 
 # ------------------------------------------------------------------------- determinism
-@pytest.mark.parametrize("name,reruns", [("C1", 100), ("C2", 10), ("C4", 3), ("C5", 5)])
+@pytest.mark.parametrize("name,reruns", [("C1", 100), ("C2", 10), ("C3", 3), ("C4", 3), ("C5", 5)])
 def test_determinism(fa, workloads, name, reruns):
     """deterministic=True is bit-identical from run to run (reference: tests/test_flash_attention_2.py:321-342)."""
     w, q, k, v, d_o = _workload_case(workloads, name)
@@ -397,6 +397,39 @@ def test_flash_attention_v2_custom_equals_default(fa, fa2_module):
         assert torch.equal(a, b), f"custom configuration differs from default for {key}"
     with pytest.raises(ValueError, match="Missing kernel configuration"):
         fa.flash_attention_v2_custom(qg, kg, vg, None, {(7, 5): configs[cc]})
+
+
+def test_custom_max_headdim_after_default_on_the_python_class(fa, fa2_module):
+    """N = 100 pads lse to 256 rows under the default max_headdim and to 128 under a custom
+    max_headdim = 128 (flash_attention_2.py:98).  Both in a row, same shapes, through the Python
+    autograd class, whose backward launcher keeps an argument record per problem: each call's
+    backward must use its own row length, and the gradients must agree bit for bit."""
+    q, k, v, d_o = _seeded((2, 3, 100, 64), (2, 3, 100, 64), torch.float16)
+    cc = torch.cuda.get_device_capability()
+    default = fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC
+    custom = fa.KernelsConfigV2(
+        block_rows_size=128, block_cols_size=64, min_block_headdim=32, max_headdim=128,
+        seqlen_cache_divisor=32, min_warps=4, max_warps=4, num_stages=2,
+        backward_autotune_configs=default.backward_autotune_configs)
+    want = oracle.naive_backward(q, k, v, d_o, None, torch.float32)
+    results = []
+    for cfg in (default, custom, default):
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        out = fa2_module.FlashAttentionV2Function.apply(qg, kg, vg, None, cfg)
+        out.backward(d_o.cuda())
+        torch.cuda.synchronize()
+        results.append((out.detach(), qg.grad, kg.grad, vg.grad))
+        for name, got, ref in zip(("o", "dq", "dk", "dv"), results[-1], want):
+            _assert_close(f"{name} (max_headdim={cfg.max_headdim})", got, ref)
+    for other in results[1:]:
+        for name, a, b in zip(("o", "dq", "dk", "dv"), results[0], other):
+            assert torch.equal(a, b), f"{name} depends on the lse padding"
+    # The same pair through the public functions (the C++ node when it is built).
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = fa.flash_attention_v2_custom(qg, kg, vg, None, {cc: custom})
+    out.backward(d_o.cuda())
+    for name, a, b in zip(("o", "dq", "dk", "dv"), results[0], (out.detach(), qg.grad, kg.grad, vg.grad)):
+        assert torch.equal(a, b), f"{name}: flash_attention_v2_custom(max_headdim=128) differs"
 
 
 def test_flash_attention_data_parallel(fa):

@@ -153,3 +153,53 @@ def test_atomic_mode_refuses_other_head_dimensions(fa2_module):
     out = fa2_module.flash_attention_v2_custom(q, q, q, None, configs)
     with pytest.raises(ValueError, match="ATOMIC_DQ"):
         out.sum().backward()
+
+
+def test_atomic_mode_from_concurrent_threads(fa2_module):
+    """Four Python threads, each on its own stream with its own problem and its own workspace (the
+    launcher allocates one per call), run the atomic backward at the same time: the only atomics in
+    the library must not mix between callers.  dK and dV must have the serial call's bits, dQ the
+    oracle's values."""
+    import threading
+
+    shapes = [(1, 2, 384, 64, torch.float16), (2, 2, 256, 128, torch.bfloat16), (1, 3, 300, 32, torch.float16),
+              (1, 2, 640, 64, torch.bfloat16)]
+    problems = [_seeded((b, h, n, d), (b, h, n, d), dt, seed=200 + i) for i, (b, h, n, d, dt) in enumerate(shapes)]
+    serial = [_run_atomic(fa2_module, *p, None) for p in problems]
+    wanted = [oracle.naive_backward(*p, None, torch.float32) for p in problems]
+    configs = {torch.cuda.get_device_capability(): fa2_module.GFX950_KERNEL_CONFIG_SEQUENCE_PARALLEL_ATOMIC}
+    rounds = 10
+    results: list = [None] * len(problems)
+    errors: list = []
+    start = threading.Barrier(len(problems))
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            q, k, v, d_o = (t.cuda() for t in problems[i])
+            torch.cuda.synchronize()
+            start.wait()
+            with torch.cuda.stream(stream):
+                for _ in range(rounds):
+                    qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
+                    out = fa2_module.flash_attention_v2_custom(qg, kg, vg, None, configs)
+                    grads = torch.autograd.grad(out, (qg, kg, vg), d_o)
+                stream.synchronize()
+            results[i] = (out.detach(),) + tuple(grads)
+        except Exception as exc:  # noqa: BLE001 - reported by the main thread
+            errors.append((i, repr(exc)))
+            start.abort()
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(problems))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for i, (got, ser, want) in enumerate(zip(results, serial, wanted)):
+        assert got is not None, f"thread {i} did not finish"
+        assert torch.equal(got[0], ser[0]), f"thread {i}: o differs from the serial call"
+        _assert_close(f"thread {i} dq", got[1], want[1])
+        for name, a, b in zip(("dk", "dv"), got[2:], ser[2:]):
+            assert torch.equal(a, b), f"thread {i}: {name} differs from the serial call"

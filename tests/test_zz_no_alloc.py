@@ -3,7 +3,7 @@
 It is called through the C ABI and compared bit for bit with fa2_bwd_fused (which gets its delta
 scratch from the caller) on two calls in a row, the second with a smaller input, so that rows the
 first call left in the library's scratch array lie beyond what the second call writes.  A third case
-goes through the generic kernels (preprocess kernel writes delta), and the size limit is checked.
+goes through the generic kernels (head dimension 50: the preprocess kernel writes delta), and the size limit is checked.
 """
 
 from __future__ import annotations
@@ -79,9 +79,13 @@ def test_noalloc_matches_fused_on_two_calls_in_a_row(capi):
 
 
 def test_noalloc_generic_kernels_and_unequal_lengths(capi):
-    # Head dimension 48 and Nq != Nk run the generic kernels: delta comes from the preprocess kernel.
-    want, got = _both_backwards(capi, 2, 2, 200, 333, 48, torch.float16, seed=3)
-    _assert_same(want, got, "generic path (B=2 H=2 Nq=200 Nk=333 D=48 fp16)")
+    # A head dimension that is not a multiple of 8 runs the generic kernels: the preprocess kernel,
+    # not the dQ kernel, writes delta into the library's scratch.
+    want, got = _both_backwards(capi, 2, 2, 200, 333, 50, torch.float16, seed=3)
+    _assert_same(want, got, "generic path (B=2 H=2 Nq=200 Nk=333 D=50 fp16)")
+    # Head dimension 48 with Nq != Nk: the padded fast kernels, delta formed inside the dQ kernel.
+    want, got = _both_backwards(capi, 2, 2, 200, 333, 48, torch.float16, seed=4)
+    _assert_same(want, got, "padded fast path (B=2 H=2 Nq=200 Nk=333 D=48 fp16)")
 
 
 def test_noalloc_refuses_sizes_beyond_its_scratch(capi):
