@@ -9,6 +9,10 @@ TFLOP/s with the FlashAttention-2 FLOP convention (fwd = 4*B*H*N^2*D/2, bwd = 2.
 the forward-only figures and fractions of the dense bf16 MFMA peak are in the same line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu-baseline]
+                    [--no-other-workloads]
+
+After the headline workload's timed region the other BASELINE configurations (and one
+short-sequence shape) are timed briefly and reported in ``other_workloads``.
 """
 
 from __future__ import annotations
@@ -284,6 +288,71 @@ def _cpu_baseline(w, workloads, heads: int):
     }
 
 
+# Workloads timed after the headline one (a few tens of milliseconds each) and reported in
+# `other_workloads`: the other four BASELINE configurations and one short-sequence, many-heads shape
+# of the kind the reference's own tests use (tests/test_flash_attention_2.py:22-29).
+OTHER_WORKLOADS = ("C1", "C2", "C4", "C5", "S512")
+
+
+def _other_workloads(pkg, workloads, dev, names, budget_ms: float = 60.0) -> dict:
+    """Forward and forward+backward time of further workloads through the same public function and
+    autograd path as the headline step.  Inputs are drawn on the device (same shapes, dtypes and
+    standard deviations as the seeded parity inputs; only timing is taken here)."""
+    table = dict(workloads.WORKLOADS)
+    table["S512"] = workloads.Workload("S512", 256, 16, 512, 64, torch.bfloat16,
+                                       description="short sequences, many heads")
+    out = {}
+    for name in names:
+        w = table[name]
+        gen = torch.Generator(device=dev).manual_seed(42)
+        q, k, v, d_o = (
+            (torch.randn(w.shape, generator=gen, device=dev, dtype=torch.float32) * std).to(w.dtype)
+            for std in (w.qk_std, w.qk_std, 1.0, 1.0))
+        q.requires_grad_(True)
+        k.requires_grad_(True)
+        v.requires_grad_(True)
+
+        def step():
+            return torch.autograd.grad(pkg.flash_attention_v2(q, k, v, w.softmax_scale, False), (q, k, v), d_o)
+
+        def fwd_only():
+            with torch.no_grad():
+                return pkg.flash_attention_v2(q, k, v, w.softmax_scale, False)
+
+        def timed(fn):
+            # Untimed calls for about a third of the budget, then as many timed calls as fit the rest.
+            fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            once_ms = max((time.perf_counter() - t0) * 1e3, 1e-3)
+            n_warm = max(3, int(budget_ms / 3 / once_ms))
+            n = max(5, min(2000, int(budget_ms * 2 / 3 / once_ms)))
+            for _ in range(n_warm):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3 / n, n
+
+        step_ms, n_step = timed(step)
+        fwd_ms, n_fwd = timed(fwd_only)
+        peak = PEAK_TFLOPS["bf16" if w.dtype == torch.bfloat16 else "f16"]
+        out[name] = {
+            "shape": list(w.shape), "dtype": "bf16" if w.dtype == torch.bfloat16 else "f16", "qk_std": w.qk_std,
+            "fwd_ms": fwd_ms, "ms_per_step": step_ms, "timed_calls": [n_fwd, n_step],
+            "fwd_tflops": w.fwd_flops / (fwd_ms * 1e-3) / 1e12,
+            "fwd_frac_of_peak": w.fwd_flops / (fwd_ms * 1e-3) / 1e12 / peak,
+            "fwd_bwd_tflops": 3.5 * w.fwd_flops / (step_ms * 1e-3) / 1e12,
+            "fwd_bwd_frac_of_peak": 3.5 * w.fwd_flops / (step_ms * 1e-3) / 1e12 / peak,
+        }
+        del q, k, v, d_o
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -298,6 +367,8 @@ def main() -> int:
     ap.add_argument("--deterministic", action="store_true", help="time the deterministic backward in the step")
     ap.add_argument("--cpu-heads", type=int, default=64, help="(batch, head) slices in the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the block of further workloads timed after the headline one")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also launch a plain 256 MiB -> 256 MiB elementwise copy three times, so a hardware-"
                          "counter run of this command holds a kernel of known HBM traffic to scale by")
@@ -470,6 +541,8 @@ def main() -> int:
         torch.cuda.synchronize()
         line["traffic_calibration"] = {"kernel": "torch elementwise mul (fp32, out=)",
                                        "read_bytes": CALIBRATION_BYTES, "write_bytes": CALIBRATION_BYTES}
+    if not args.no_other_workloads:
+        line["other_workloads"] = _other_workloads(pkg, workloads, dev, [n for n in OTHER_WORKLOADS if n != w.name])
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(w, workloads, args.cpu_heads)
     print(json.dumps(line))

@@ -15,7 +15,7 @@ import threading
 # The in-tree build; FA2_GFX950_LIBRARY names another build of the same ABI (e.g. one under test).
 LIBRARY_PATH = pathlib.Path(os.environ.get("FA2_GFX950_LIBRARY") or
                             pathlib.Path(__file__).resolve().parent / "csrc" / "libfa2_gfx950.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 FA2_DTYPE_F16 = 0
 FA2_DTYPE_BF16 = 1
@@ -35,7 +35,7 @@ class ConfigInfo(ctypes.Structure):
         "bwd_block_q", "bwd_block_kv", "bwd_waves",
         "dq_block_q", "dq_block_kv", "dq_waves",
         "lds_direct", "fwd_wg_per_cu", "dq_wg_per_cu", "dkdv_wg_per_cu",
-        "lds_stages", "dkdv_passes", "head_group", "dq_atomic")]
+        "lds_stages", "dkdv_passes", "head_group", "dq_atomic", "fwd_exp_folded")]
 
     def as_dict(self) -> dict:
         return {name: getattr(self, name) for name, _ in self._fields_}
@@ -74,6 +74,7 @@ SIGNATURES = {
     "fa2_config_count": (_i, []),
     "fa2_config_get": (_i, [_i, ctypes.POINTER(ConfigInfo)]),
     "fa2_pick_config": (_i, [_i, _i, _i, _i, _i]),
+    "fa2_pick_config_forward_only": (_i, [_i, _i, _i, _i]),
     "fa2_fwd": (_i, [_p] * 5 + [_i] * 6 + [_i64] * 12 + [_f, _i, _i, _p]),
     "fa2_bwd_preprocess": (_i, [_p] * 3 + [_i] * 5 + [_i64] * 6 + [_i, _p]),
     "fa2_bwd_workspace_bytes": (ctypes.c_size_t, [_i] * 7),

@@ -8,8 +8,8 @@ per padded head dimension, chosen by the library from the problem), so of the fi
 ``max_headdim`` (largest accepted head dimension, padding of the log-sum-exp rows), the
 ``SEQUENCE_PARALLEL`` flag of the backward configurations (which backward mode is requested) and,
 next to it, ``ATOMIC_DQ`` (run the reference's atomic-add formulation of that mode, see
-``KernelsConfigV2.atomic_dq``) have an effect; the Triton tile, warp and stage counts are accepted
-and ignored.  The reference's
+``KernelsConfigV2.atomic_dq``) have an effect, plus one field the reference does not have,
+``exact_scale``; the Triton tile, warp and stage counts are accepted and ignored.  The reference's
 kernel-cache key helpers (_configurators_v2.py:40-78) have no counterpart: there is no run-time
 compilation and therefore no kernel cache to key.
 """
@@ -60,6 +60,12 @@ class KernelsConfigV2:
         num_stages: LDS stages of the streamed tiles (compiled: 2).
         backward_autotune_configs: Backward configurations; the backward is deterministic
             unless one of them sets ``SEQUENCE_PARALLEL`` to True.
+        exact_scale: Not in the reference.  A forward that nothing will differentiate may, for bf16
+            inputs, run a kernel that multiplies Q by ``softmax_scale * log2(e)`` and rounds it to
+            bf16 once (table rows with ``fwd_exp_folded``); True keeps such calls on the rows that
+            apply the scale to the fp32 scores, as the reference does
+            (_triton_kernels_v2.py:137-152), at about 4 % more forward time.  Forwards that a
+            backward may follow, and fp16 inputs, always take those rows.
     """
 
     block_rows_size: int
@@ -71,6 +77,7 @@ class KernelsConfigV2:
     max_warps: int
     num_stages: int
     backward_autotune_configs: list = field(default_factory=list)
+    exact_scale: bool = False
 
     @property
     def deterministic(self) -> bool:

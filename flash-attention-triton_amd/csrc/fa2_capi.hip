@@ -44,21 +44,31 @@ constexpr int kHeadGroup = 64;
 constexpr int kHeadGroup128 = 32;
 
 const fa2_config_info kTable[] = {
-    // id DP  fwd:BQ       BKV        waves dK/dV:BQ   BKV       waves dQ:BQ    BKV      waves fast fwd/CU dq/CU dkdv/CU stages passes group
-    {0, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 4, 3, 3, 1, kHeadGroup, 0},
-    {1, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 3, 2, 3, 1, kHeadGroup, 0},
-    {2, 96, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup, 0},
-    {3, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup128, 0},
-    {4, 192, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 2, 1, 1, 1, 2, 1, kHeadGroup, 0},
-    {5, 256, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 2, 1, 1, 1, 2, 2, kHeadGroup, 0},
+    // id DP  fwd:BQ       BKV        waves dK/dV:BQ   BKV       waves dQ:BQ    BKV      waves fast fwd/CU dq/CU dkdv/CU stages passes group atomic folded
+    {0, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 4, 3, 3, 1, kHeadGroup, 0, 0},
+    {1, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 3, 2, 3, 1, kHeadGroup, 0, 0},
+    {2, 96, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup, 0, 0},
+    {3, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup128, 0, 0},
+    {4, 192, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 2, 1, 1, 1, 2, 1, kHeadGroup, 0, 0},
+    {5, 256, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 2, 1, 1, 1, 2, 2, kHeadGroup, 0, 0},
     // Sequence-parallel rows (dq_atomic = 1): the backward is one key-tile-parallel kernel that adds its
     // dQ contributions into an fp32 workspace with global atomics, the reference's non-deterministic
     // formulation (_triton_kernels_v2.py:336-339).  Never picked automatically: on MI355X the atomics
     // alone take longer than the whole two-kernel backward (profiles/bwd_sequence_parallel_atomic_*.txt);
     // a caller selects them by id.  Forward columns as in the row of the same head dimension.
-    {6, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 0, 1, 3, 1, kHeadGroup, 1},
-    {7, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 0, 1, 3, 1, kHeadGroup, 1},
-    {8, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 0, 1, 3, 1, kHeadGroup128, 1},
+    {6, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 0, 1, 3, 1, kHeadGroup, 1, 0},
+    {7, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 0, 1, 3, 1, kHeadGroup, 1, 0},
+    {8, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 0, 1, 3, 1, kHeadGroup128, 1, 0},
+    // Forward-only rows (fwd_exp_folded = 1): as rows 0-3, with the LDS-direct forward taking its exponents
+    // straight from the score MFMAs (Q fragments multiplied by scale * log2(e) and rounded once).  Forward
+    // -4 % on B=2 H=32 N=4096 D=128, -5 % at N=16384, -3.7 % at D=64.  Never picked by FA2_CONFIG_AUTO and
+    // refused by the backward, which recomputes the probabilities from Q itself and needs the log-sum-exp
+    // of exactly those scores; fa2_pick_config_forward_only returns them for bf16, where the extra half
+    // unit in the last place of Q is of the size of the rounding the inputs already carry.
+    {9, 32, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 4, 4, 3, 3, 1, kHeadGroup, 0, 1},
+    {10, 64, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 3, 3, 2, 3, 1, kHeadGroup, 0, 1},
+    {11, 96, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup, 0, 1},
+    {12, 128, kFwdBlockQ, kFwdBlockKV, 4, kDkvBlockQ, kDkvBlockKV, 4, kDqBlockQ, kDqBlockKV, 4, 1, 2, 2, 1, 3, 1, kHeadGroup128, 0, 1},
 };
 constexpr int kTableRows = sizeof(kTable) / sizeof(kTable[0]);
 
@@ -66,10 +76,21 @@ constexpr int kTableRows = sizeof(kTable) / sizeof(kTable[0]);
 // the heads there are (fa2::equal_head_groups).
 int head_group(int cfg, int64_t heads) { return fa2::equal_head_groups(kTable[cfg].head_group, heads); }
 
+// The row FA2_CONFIG_AUTO stands for: the first plain row wide enough for the head dimension.
 int pick_config(int headdim) {
   for (int i = 0; i < kTableRows; i++)
-    if (!kTable[i].dq_atomic && headdim <= kTable[i].headdim_padded) return i;
+    if (!kTable[i].dq_atomic && !kTable[i].fwd_exp_folded && headdim <= kTable[i].headdim_padded) return i;
   return -1;
+}
+
+// The row for a forward whose log-sum-exp no backward will read: for bf16 the folded row of the
+// head dimension when there is one, else the plain row.
+int pick_config_forward_only(int dtype, int headdim) {
+  const int plain = pick_config(headdim);
+  if (plain < 0 || dtype != FA2_DTYPE_BF16) return plain;
+  for (int i = 0; i < kTableRows; i++)
+    if (kTable[i].fwd_exp_folded && kTable[i].headdim_padded == kTable[plain].headdim_padded) return i;
+  return plain;
 }
 
 // Query rows of the fp32 dQ accumulator of a sequence-parallel row: whole 64-row query tiles.
@@ -165,8 +186,8 @@ int fwd_impl(const fa2_fwd_args &a, void *stream) {
 
   const int64_t nwg = (int64_t)p.n_qtiles * a.batch * a.nheads;
   if (nwg > 0x7fffffff) return fail(FA2_ERR_TOO_LARGE, "grid of %lld workgroups too large", (long long)nwg);
-  fa2::launch_fwd(a.dtype == FA2_DTYPE_BF16, kTable[cfg].headdim_padded, p, dim3((unsigned)nwg),
-                  reinterpret_cast<hipStream_t>(stream));
+  fa2::launch_fwd(a.dtype == FA2_DTYPE_BF16, kTable[cfg].headdim_padded, kTable[cfg].fwd_exp_folded != 0, p,
+                  dim3((unsigned)nwg), reinterpret_cast<hipStream_t>(stream));
   return launch_status("fa2_fwd launch");
 }
 
@@ -230,6 +251,9 @@ int bwd_impl(const fa2_bwd_args &a, void *stream) {
     return fail(FA2_ERR_BAD_SHAPE, "softmax_scale must be positive and finite, got %g", (double)a.softmax_scale);
   int cfg;
   if ((rc = resolve_config(a.config_id, a.headdim, &cfg))) return rc;
+  if (kTable[cfg].fwd_exp_folded)
+    return fail(FA2_ERR_BAD_CONFIG, "config %d is a forward-only row: its forward rounds Q * scale, and the "
+                                    "backward recomputes the probabilities from Q itself", cfg);
 
   p.lse = a.lse;
   p.delta = a.delta;
@@ -384,7 +408,7 @@ int fa2_config_get(int config_id, fa2_config_info *out) {
 }
 
 int fa2_pick_config(int dtype, int headdim, int seqlen_q, int seqlen_k, int deterministic) {
-  (void)deterministic;  // both backward modes use the same row
+  (void)deterministic;  // both backward modes use the same row; sequence lengths are validated only
   if (dtype != FA2_DTYPE_F16 && dtype != FA2_DTYPE_BF16)
     return -fail(FA2_ERR_BAD_DTYPE, "dtype %d is neither FA2_DTYPE_F16 nor FA2_DTYPE_BF16", dtype);
   if (headdim <= 0 || seqlen_q <= 0 || seqlen_k <= 0)
@@ -394,6 +418,11 @@ int fa2_pick_config(int dtype, int headdim, int seqlen_q, int seqlen_k, int dete
   if (id < 0)
     return -fail(FA2_ERR_HEADDIM, "Supports head dimensions only up to %d, got %d", FA2_MAX_HEADDIM, headdim);
   return id;
+}
+
+int fa2_pick_config_forward_only(int dtype, int headdim, int seqlen_q, int seqlen_k) {
+  const int id = fa2_pick_config(dtype, headdim, seqlen_q, seqlen_k, 0);  // validates
+  return id < 0 ? id : pick_config_forward_only(dtype, headdim);
 }
 
 int fa2_fwd_packed(const fa2_fwd_args *args, void *stream) {

@@ -130,6 +130,15 @@ __device__ __forceinline__ float sum_over_halves(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Eight half-precision values times a constant, rounded back to half precision.
+template <typename T>
+__device__ __forceinline__ s16x8 scale8(s16x8 x, float mult) {
+  f32x8 f;
+#pragma unroll
+  for (int j = 0; j < 8; j++) f[j] = Elem<T>::to_float(x[j]) * mult;
+  return Elem<T>::pack8(f);
+}
+
 // Sixteen copies of one value, kept in sixteen registers: the form an MFMA takes as its C operand.
 // The empty asm statement hides from the optimiser that the registers are equal; otherwise it
 // rebuilds the block with sixteen moves in front of every use.
@@ -304,6 +313,13 @@ __device__ __forceinline__ void load_lds_16(const short *uniform_base, unsigned 
 
 // s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt fields left at their maxima).
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// s_waitcnt vmcnt(N) only, 0 <= N < 64: wait until at most N vector-memory loads of this wave are
+// outstanding (vmcnt is split in the gfx9 encoding: bits 3:0 and 15:14).
+template <int N>
+__device__ __forceinline__ void wait_vmem() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
 
 // Row pitch, in elements, of the LDS tiles of the fast kernels for head dimension DP.  The swizzle
 // needs a power-of-two number of 16-byte chunks per row, so 96 columns live in rows of 128: the

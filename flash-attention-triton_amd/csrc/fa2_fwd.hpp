@@ -296,7 +296,11 @@ struct HalfTag {
 
 // PAD: the head dimension is a multiple of 8 below DP; the columns beyond it are zeros in LDS and in
 // the register fragments, and are not stored.
-template <typename T, int DP, int BKV, bool PAD>
+// PRE: the Q fragments are multiplied by scale * log2(e) and rounded to half precision once, and
+// every score chain starts from minus the maximum in use (the MFMA's C operand), so that the score
+// MFMAs deliver the base-2 exponents themselves and no multiply-add is left in front of the
+// exponentials.
+template <typename T, int DP, int BKV, bool PAD, bool PRE>
 __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direct_kernel(const FwdParams p) {
   using L = FwdDirectLayout<DP, BKV>;
   constexpr int KS = DP / 16, DB = DP / 32, LP = L::LP;
@@ -353,20 +357,22 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
     const unsigned dst = lds_base + 2u * (unsigned)(L::V_BASE + (t % L::V_STAGES) * L::TILE_ELEMS);
     if (t < n_inside) vload.issue(t * BKV, dst); else vload.issue_clamped(t * BKV, seqlen_k, dst);
   };
-  // K_0, V_0 and K_1 are loaded here; after that tile t brings in K_{t+2} and V_{t+1}.
+  // K_0, the workgroup's Q rows, V_0 and K_1 are loaded here; after that tile t brings in K_{t+2}
+  // and V_{t+1}.  The Q rows travel like a K tile: coalesced LDS-direct loads (a wave-load covers
+  // whole rows) into the two stages nothing else uses yet, query rows 0..63 of the workgroup in
+  // the third K stage and 64..127 in the second V stage, from where every wave reads its
+  // fragments.  Loaded straight into registers, a wave's fragment loads touch 32 different rows
+  // each, eight times over, and keep the CU's address path busy for a microsecond per workgroup.
+  // Rows beyond the sequence are read from its last row: finite values whose results are never stored.
+  constexpr unsigned Q_LO = 2u * (unsigned)(L::K_BASE + 2 * L::TILE_ELEMS);
+  constexpr unsigned Q_HI = 2u * (unsigned)(L::V_BASE + 1 * L::TILE_ELEMS);
+  const TileLoader<DP, BKV, kFwdWaves, PAD> qload(Q + (int64_t)q0 * p.q.stride_seq, p.q.stride_seq, hdim / 8);
+  const int q_rows = p.seqlen_q - q0;  // rows of this query tile that exist (>= 1)
   issue_k(0);
+  if (q_rows >= BKV) qload.issue(0, lds_base + Q_LO); else qload.issue_clamped(0, q_rows, lds_base + Q_LO);
+  if (q_rows >= 2 * BKV) qload.issue(BKV, lds_base + Q_HI); else qload.issue_clamped(BKV, q_rows, lds_base + Q_HI);
   issue_v(0);
   if (n_tiles > 1) issue_k(1);
-
-  // Q^T fragments (B operand of S^T = K Q^T): lane (c, h) holds Q[q0w + c][16 ks + 8 h + j].
-  s16x8 qf[KS];
-  {
-    const int row = q0w + c;
-    const bool ok = row < p.seqlen_q;
-    const short *rp = Q + (int64_t)row * p.q.stride_seq;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[ks] = load_chunk(rp, 16 * ks + 8 * h, hdim, ok, true);
-  }
 
   // Fragment addresses (swizzled, 32-bit LDS pointers).  kcur points into the stage of the K tile
   // after the current one, vcur into the stage of the current V tile; both advance by a uniform
@@ -399,7 +405,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
   for (int db = 0; db < DB; db++)
 #pragma unroll
     for (int i = 0; i < 16; i++) oacc[db][i] = 0.f;
-  float m_ref = -INFINITY;  // maximum (raw scores) the probabilities are formed against
+  float m_ref = -INFINITY;  // maximum the probabilities are formed against (raw scores; PRE: base-2 exponents)
   float l_run = 0.f;        // this lane's share of the running sum (its half of the key rows)
   const int qrow = q0w + c;
   const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -417,8 +423,25 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
     for (int i = 1; i < 16; i++) m = fmaxf(m, s[i]);
     return max_over_halves(m);
   };
-  wait_vmem_all();
+  // K_0 and Q have landed once at most the loads of V_0 (and K_1) are outstanding: loads complete
+  // in the order they were issued.
+  constexpr int LOADS_PER_TILE = TileLoader<DP, BKV, kFwdWaves, PAD>::LOADS;
+  static_assert(2 * LOADS_PER_TILE < 64, "vmcnt field");
+  if (n_tiles > 1) wait_vmem<2 * LOADS_PER_TILE>(); else wait_vmem<LOADS_PER_TILE>();
   __syncthreads();
+
+  // Q^T fragments (B operand of S^T = K Q^T): lane (c, h) holds Q[q0w + c][16 ks + 8 h + j].
+  s16x8 qf[KS];
+  {
+    const lds_cptr qrows = lds0 + ((wave >> 1) ? (int)(Q_HI / 2) : (int)(Q_LO / 2));
+    const int r = 32 * (wave & 1) + c;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = lds_read_128(qrows + swz_off<LP>(r, 2 * ks + h));
+    if (PRE) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) qf[ks] = scale8<T>(qf[ks], scale_log2);
+    }
+  }
 
   // ---- prologue: S_0, its row maximum, e_0 = exp2(scale*S_0 - scale*m), ring <- K fragments of
   // block 1 ---------------------------------------------------------------------------------
@@ -436,7 +459,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
     const float mc = m_ref * scale_log2;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-      e[i] = fast_exp2(sc[i] * scale_log2 - mc);
+      e[i] = PRE ? fast_exp2(sc[i] - m_ref) : fast_exp2(sc[i] * scale_log2 - mc);
       l_run += e[i];
     }
 #pragma unroll
@@ -445,6 +468,14 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) kcur[ks] += L::TILE_ELEMS;
   }
+  // V_0 and K_1 have landed, and every wave has taken its Q fragments out of the two stages that
+  // the first tile's loads (K_2, V_1) are about to overwrite.
+  wait_vmem_all();
+  __syncthreads();
+
+  // PRE: the C operand every later score chain starts from.
+  f32x16 negm = zero;
+  if (PRE) negm = splat16(-m_ref);
 
   // One block step.  On entry e holds the probabilities of block j (formed against m_ref) and the
   // ring the K fragments of block j+1.
@@ -489,10 +520,10 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
     const unsigned vdst = lds_base + 2u * (unsigned)(L::V_BASE + (vt % L::V_STAGES) * L::TILE_ELEMS);
     typedef unsigned u32x4v __attribute__((ext_vector_type(4)));
     u32x4v w[2];  // packed probabilities, two per word: w[0] = k-step 0, w[1] = k-step 1
-    sc = zero;
+    if (!PRE) sc = zero;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      sc = Elem<T>::mfma(ring[ks], qf[ks], sc);
+      sc = Elem<T>::mfma(ring[ks], qf[ks], (PRE && ks == 0) ? negm : sc);
       if (SPREAD && ks % LOAD_EVERY == 0 && ks / LOAD_EVERY < LOADS) vload.issue_one(vt * BKV, vdst, ks / LOAD_EVERY);
       ring[ks] = v_frag(HALF, ks / DB, ks % DB);
 #pragma unroll
@@ -520,7 +551,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
         ring[slot] = k_frag(HALF, slot);
 #pragma unroll
         for (int i = part(16, KS, slot); i < part(16, KS, slot + 1); i++) {
-          e[i] = fast_exp2(sc[i] * scale_log2 - mc);
+          e[i] = PRE ? fast_exp2(sc[i]) : fast_exp2(sc[i] * scale_log2 - mc);
           lsum[i & 1] += e[i];
         }
         asm volatile("" : "+v"(lsum[0]), "+v"(lsum[1]));
@@ -535,9 +566,12 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
       float lblk = lsum[0] + lsum[1];
       const bool grow = !(lblk <= kSumTrigger);
       if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-        const float m_new = fmaxf(m_ref, row_max(sc));
-        const float alpha = fast_exp2((m_ref - m_new) * scale_log2);
+        // PRE: sc holds the exponents relative to m_ref; raise m_ref by the largest positive excess.
+        const float up = fmaxf(row_max(sc), 0.f);
+        const float m_new = PRE ? m_ref + up : fmaxf(m_ref, row_max(sc));
+        const float alpha = PRE ? fast_exp2(-up) : fast_exp2((m_ref - m_new) * scale_log2);
         m_ref = m_new;
+        if (PRE) negm = splat16(-m_ref);
         l_run *= alpha;
 #pragma unroll
         for (int db = 0; db < DB; db++)
@@ -547,7 +581,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
         lblk = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          e[i] = fast_exp2(sc[i] * scale_log2 - mc2);
+          e[i] = PRE ? fast_exp2(sc[i] - up) : fast_exp2(sc[i] * scale_log2 - mc2);
           lblk += e[i];
         }
       }
@@ -589,7 +623,7 @@ __global__ __launch_bounds__(64 * kFwdWaves, (DP <= 128 ? 2 : 1)) void fwd_direc
   }
   const float l_tot = sum_over_halves(l_run);
   const float inv_l = 1.f / l_tot;
-  if (h == 0 && q0w + c < p.seqlen_q) LSE[q0w + c] = m_ref * p.scale + __logf(l_tot);
+  if (h == 0 && q0w + c < p.seqlen_q) LSE[q0w + c] = m_ref * (PRE ? kLn2 : p.scale) + __logf(l_tot);
   if (qt == p.n_qtiles - 1) {
     for (int r = p.seqlen_q + tid; r < p.seqlen_q_rounded; r += NTHREADS) LSE[r] = 0.f;
   }

@@ -17,26 +17,30 @@ void launch_generic(int dp, const FwdParams &p, dim3 grid, dim3 block, hipStream
   }
 }
 
-template <typename T, bool PAD>
+// PRE (exponents straight from the score MFMAs) is instantiated up to 128 columns: the sixteen registers
+// of the chain's start value are more than the 256-column kernel has left.
+template <typename T, bool PAD, bool PRE>
 void launch_direct(int dp, const FwdParams &p, dim3 grid, dim3 block, hipStream_t s) {
   switch (dp) {
-    case 32: hipLaunchKernelGGL((fwd_direct_kernel<T, 32, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
-    case 64: hipLaunchKernelGGL((fwd_direct_kernel<T, 64, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
-    case 96: hipLaunchKernelGGL((fwd_direct_kernel<T, 96, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
-    case 128: hipLaunchKernelGGL((fwd_direct_kernel<T, 128, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
-    case 192: hipLaunchKernelGGL((fwd_direct_kernel<T, 192, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fwd_direct_kernel<T, 256, kFwdBlockKV, PAD>), grid, block, 0, s, p); break;
+    case 32: hipLaunchKernelGGL((fwd_direct_kernel<T, 32, kFwdBlockKV, PAD, PRE>), grid, block, 0, s, p); break;
+    case 64: hipLaunchKernelGGL((fwd_direct_kernel<T, 64, kFwdBlockKV, PAD, PRE>), grid, block, 0, s, p); break;
+    case 96: hipLaunchKernelGGL((fwd_direct_kernel<T, 96, kFwdBlockKV, PAD, PRE>), grid, block, 0, s, p); break;
+    case 128: hipLaunchKernelGGL((fwd_direct_kernel<T, 128, kFwdBlockKV, PAD, PRE>), grid, block, 0, s, p); break;
+    case 192: hipLaunchKernelGGL((fwd_direct_kernel<T, 192, kFwdBlockKV, PAD, false>), grid, block, 0, s, p); break;
+    default: hipLaunchKernelGGL((fwd_direct_kernel<T, 256, kFwdBlockKV, PAD, false>), grid, block, 0, s, p); break;
   }
 }
 
 template <typename T>
-void launch(int dp, const FwdParams &p, dim3 grid, hipStream_t s) {
+void launch(int dp, bool folded, const FwdParams &p, dim3 grid, hipStream_t s) {
   const dim3 block(64 * kFwdWaves);
   if (fwd_direct_ok(dp, p)) {
-    if (p.headdim == dp)
-      launch_direct<T, false>(dp, p, grid, block, s);
-    else
-      launch_direct<T, true>(dp, p, grid, block, s);
+    const bool pad = p.headdim != dp;
+    if (folded) {
+      if (pad) launch_direct<T, true, true>(dp, p, grid, block, s); else launch_direct<T, false, true>(dp, p, grid, block, s);
+    } else {
+      if (pad) launch_direct<T, true, false>(dp, p, grid, block, s); else launch_direct<T, false, false>(dp, p, grid, block, s);
+    }
     return;
   }
   if (p.vec)
@@ -47,11 +51,11 @@ void launch(int dp, const FwdParams &p, dim3 grid, hipStream_t s) {
 
 }  // namespace
 
-void launch_fwd(bool bf16, int dp, const FwdParams &p, dim3 grid, hipStream_t s) {
+void launch_fwd(bool bf16, int dp, bool folded, const FwdParams &p, dim3 grid, hipStream_t s) {
   if (bf16)
-    launch<__bf16>(dp, p, grid, s);
+    launch<__bf16>(dp, folded, p, grid, s);
   else
-    launch<_Float16>(dp, p, grid, s);
+    launch<_Float16>(dp, folded, p, grid, s);
 }
 
 }  // namespace fa2

@@ -26,7 +26,8 @@ inline bool direct_headdim_kv_stream(int dp, int headdim) {
   return direct_headdim(dp, headdim) || (headdim % 8 == 0 && headdim <= dp && (dp == 192 || dp == 256));
 }
 inline bool fwd_direct_ok(int dp, const FwdParams &p) {
-  return p.vec && direct_headdim_kv_stream(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
+  return p.vec && direct_headdim_kv_stream(dp, p.headdim) && direct_stride_ok(p.q) && direct_stride_ok(p.k) &&
+         direct_stride_ok(p.v);
 }
 inline bool dq_direct_ok(int dp, const BwdParams &p) {
   return p.vec && direct_headdim_kv_stream(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
@@ -53,7 +54,9 @@ inline int equal_head_groups(int group, int64_t heads) {
 }
 
 // bf16 != 0 selects the bf16 kernels, otherwise fp16.
-void launch_fwd(bool bf16, int dp, const FwdParams &p, dim3 grid, hipStream_t s);
+// folded: the LDS-direct forward takes its exponents straight from the score MFMAs (Q fragments
+// multiplied by scale * log2(e) and rounded once); the generic forward ignores it.
+void launch_fwd(bool bf16, int dp, bool folded, const FwdParams &p, dim3 grid, hipStream_t s);
 void launch_preprocess(bool bf16, const PreParams &p, dim3 grid, hipStream_t s);
 // fuse_delta: the fast dQ kernel also forms delta from O and dO (dq_direct_ok must hold).
 void launch_dq(bool bf16, int dp, const BwdParams &p, dim3 grid, bool fuse_delta, hipStream_t s);

@@ -48,7 +48,7 @@ struct FlashAttentionV2 : public torch::autograd::Function<FlashAttentionV2> {
   // softmax_scale > 0 (the wrapper folds a negative scale into the sign of q).
   static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &q, const at::Tensor &k,
                             const at::Tensor &v, double softmax_scale, bool deterministic,
-                            int64_t max_headdim) {
+                            int64_t max_headdim, bool forward_only) {
     const c10::DeviceGuard guard(q.device());
     const int64_t batch = q.size(0), nheads = q.size(1), seqlen_q = q.size(2), headdim = q.size(3);
     const int64_t seqlen_k = k.size(2);
@@ -70,7 +70,10 @@ struct FlashAttentionV2 : public torch::autograd::Function<FlashAttentionV2> {
     a.seqlen_q_rounded = (int)seqlen_q_rounded;
     a.softmax_scale = (float)softmax_scale;
     a.dtype = dtype_code(q);
-    a.config_id = FA2_CONFIG_AUTO;
+    // forward_only: the caller knows that nothing will be differentiated, so no backward reads lse.
+    a.config_id = forward_only ? fa2_pick_config_forward_only(a.dtype, a.headdim, a.seqlen_q, a.seqlen_k)
+                               : FA2_CONFIG_AUTO;
+    if (forward_only && a.config_id < 0) check(-a.config_id, "fa2_pick_config_forward_only");
     check(fa2_fwd_packed(&a, current_stream(q)), "fa2_fwd");
 
     ctx->save_for_backward({q, k, v, o, lse});
@@ -117,13 +120,13 @@ struct FlashAttentionV2 : public torch::autograd::Function<FlashAttentionV2> {
     a.deterministic = ctx->saved_data["deterministic"].toBool() ? 1 : 0;
     a.config_id = FA2_CONFIG_AUTO;
     check(fa2_bwd_packed(&a, current_stream(q)), "fa2_bwd");
-    return {dq, dk, dv, at::Tensor(), at::Tensor(), at::Tensor()};
+    return {dq, dk, dv, at::Tensor(), at::Tensor(), at::Tensor(), at::Tensor()};
   }
 };
 
 at::Tensor flash_attention_v2(const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
-                              double softmax_scale, bool deterministic, int64_t max_headdim) {
-  return FlashAttentionV2::apply(q, k, v, softmax_scale, deterministic, max_headdim);
+                              double softmax_scale, bool deterministic, int64_t max_headdim, bool forward_only) {
+  return FlashAttentionV2::apply(q, k, v, softmax_scale, deterministic, max_headdim, forward_only);
 }
 
 }  // namespace
@@ -133,6 +136,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("flash_attention_v2", &flash_attention_v2,
         "q, k, v: contiguous CUDA fp16/bf16 (B, H, N, D); softmax_scale > 0; returns o",
         py::arg("q"), py::arg("k"), py::arg("v"), py::arg("softmax_scale"), py::arg("deterministic"),
-        py::arg("max_headdim"));
+        py::arg("max_headdim"), py::arg("forward_only") = false);
   m.def("abi_version", []() { return fa2_abi_version(); });
 }

@@ -11,6 +11,14 @@ Differences from the reference, all deliberate:
   (flash_attention_2.py:316).  fp16 inputs use fp16 MFMA; any other dtype is down-cast to fp16
   and the output cast back, as in the reference.
 * fp16/bf16 contiguous inputs are used as they are: no cast or copy kernels run.
+* A forward that nothing will differentiate (under ``torch.no_grad()``, or with no input that
+  requires a gradient) on bf16 inputs up to head dimension 128 multiplies Q by
+  softmax_scale * log2(e) and rounds it to bf16 once, so that the score MFMAs deliver base-2
+  exponents (4 % less time; the reference scales the fp32 scores, _triton_kernels_v2.py:137-152).
+  Whenever a backward may follow, and always for fp16, the forward uses the reference's arithmetic:
+  the backward recomputes the probabilities from Q itself and needs the log-sum-exp of exactly those
+  scores.  ``KernelsConfigV2.exact_scale`` (through ``flash_attention_v2_custom``) or
+  ``FA2_GFX950_EXACT_SCALE=1`` keeps the reference's arithmetic everywhere.
 * The configuration selector knows one architecture, gfx950.
 * ``deterministic=True`` does not serialise the backward into one program per head
   (flash_attention_2.py:204-207): dQ is produced by a query-tile-parallel kernel that accumulates
@@ -115,12 +123,15 @@ def _flash_attention_forward(
     min_warps: int,
     max_warps: int,
     num_stages: int,
+    forward_only: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor, float]:
     """Validate inputs, allocate O and the log-sum-exp, launch the forward kernel.
 
     Same signature, checks and return value as the reference launcher
     (flash_attention_2.py:61-144).  The tile arguments are accepted for compatibility; the tile
-    shape comes from the table inside the library.
+    shape comes from the table inside the library.  ``forward_only`` (not in the reference) says
+    that no backward will read the log-sum-exp: the library may then pick a row whose forward folds
+    the softmax scale into Q (``fa2_pick_config_forward_only``; bf16 up to head dimension 128).
     """
     batch, nheads, seqlen_q, headdim = q.shape
     _, _, seqlen_k, _ = k.shape
@@ -140,8 +151,9 @@ def _flash_attention_forward(
 
     # One argument record per (shapes, strides, dtype, scale), kept between calls: only the five
     # pointers change from call to call.
+    config_id = _forward_only_row(q.dtype, headdim, seqlen_q, seqlen_k) if forward_only else _capi.FA2_CONFIG_AUTO
     key = (q_in.shape, seqlen_k, q_in.stride(), k.stride(), v.stride(), output.stride(), q.dtype,
-           seqlen_q_rounded, kernel_scale, threading.get_ident())
+           seqlen_q_rounded, kernel_scale, config_id, threading.get_ident())
     args = _FWD_ARGS.get(key)
     if args is None:
         args = _capi.FwdArgs()
@@ -151,7 +163,7 @@ def _flash_attention_forward(
         args.batch, args.nheads, args.seqlen_q, args.seqlen_k = batch, nheads, seqlen_q, seqlen_k
         args.headdim, args.seqlen_q_rounded = headdim, seqlen_q_rounded
         args.softmax_scale, args.dtype = kernel_scale, _COMPUTE_DTYPES[q.dtype]
-        args.config_id = _capi.FA2_CONFIG_AUTO
+        args.config_id = config_id
         _remember(_FWD_ARGS, key, args)
     args.q.ptr, args.k.ptr, args.v.ptr = q_in.data_ptr(), k.data_ptr(), v.data_ptr()
     args.o.ptr, args.lse = output.data_ptr(), lse.data_ptr()
@@ -252,6 +264,25 @@ def _flash_attention_backward(
         dq.neg_()
 
 
+# FA2_GFX950_EXACT_SCALE=1 keeps forward-only calls on the rows of the reference's arithmetic too.
+_EXACT_SCALE_ONLY = bool(os.environ.get("FA2_GFX950_EXACT_SCALE"))
+_FORWARD_ONLY_ROWS: dict = {}
+
+
+def _forward_only_row(dtype: torch.dtype, headdim: int, seqlen_q: int, seqlen_k: int) -> int:
+    """Table row for a forward whose log-sum-exp no backward will read."""
+    if _EXACT_SCALE_ONLY:
+        return _capi.FA2_CONFIG_AUTO
+    key = (dtype, headdim)
+    row = _FORWARD_ONLY_ROWS.get(key)
+    if row is None:
+        row = _capi.load().fa2_pick_config_forward_only(_COMPUTE_DTYPES[dtype], headdim, seqlen_q, seqlen_k)
+        if row < 0:
+            _capi.check(-row, "fa2_pick_config_forward_only")
+        _FORWARD_ONLY_ROWS[key] = row
+    return row
+
+
 _ATOMIC_ROWS: dict[int, int] = {}
 
 
@@ -297,6 +328,9 @@ class FlashAttentionV2Function(torch.autograd.Function):
             kernels_config.min_warps,
             kernels_config.max_warps,
             kernels_config.num_stages,
+            # Nothing will be differentiated (no_grad, or no input that requires a gradient): the
+            # log-sum-exp saved below is never read.
+            forward_only=not any(ctx.needs_input_grad[:3]) and not getattr(kernels_config, "exact_scale", False),
         )
 
         ctx.save_for_backward(q, k, v, output, lse)
@@ -366,7 +400,7 @@ def _apply(q, k, v, softmax_scale, kernels_config):  # noqa: ANN001, ANN202
     checks are the launcher's, a negative scale is folded into the sign of q.
     """
     node = _cpp_node()
-    if node is None or kernels_config.atomic_dq:  # the C++ node always lets the table choose
+    if node is None or kernels_config.atomic_dq:  # the C++ node always lets the table choose its backward row
         return FlashAttentionV2Function.apply(q, k, v, softmax_scale, kernels_config)
     initial_dtype = q.dtype
     compute_dtype = _compute_dtype(initial_dtype)
@@ -377,7 +411,11 @@ def _apply(q, k, v, softmax_scale, kernels_config):  # noqa: ANN001, ANN202
     scale = softmax_scale or 1.0 / math.sqrt(q.shape[-1])
     if scale < 0:
         q, scale = -q, -scale
-    output = node.flash_attention_v2(q, k, v, scale, bool(kernels_config.deterministic), kernels_config.max_headdim)
+    # A forward that nothing will differentiate may take a forward-only row of the table.
+    forward_only = (not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad))
+                    and not getattr(kernels_config, "exact_scale", False) and not _EXACT_SCALE_ONLY)
+    output = node.flash_attention_v2(q, k, v, scale, bool(kernels_config.deterministic), kernels_config.max_headdim,
+                                     forward_only)
     return output if initial_dtype == compute_dtype else output.to(initial_dtype)
 
 
@@ -546,9 +584,9 @@ def flash_attention_v2_custom(
 
     Same contract as the reference (flash_attention_2.py:700-790): the dictionary is keyed by
     ``torch.cuda.get_device_capability()`` of the current device ((9, 5) on MI355X); a missing
-    key raises ValueError.  Of the configuration, ``max_headdim`` and the ``SEQUENCE_PARALLEL``
-    and ``ATOMIC_DQ`` flags of the backward configurations are honoured (the latter selects the
-    atomic-add backward, ``GFX950_KERNEL_CONFIG_SEQUENCE_PARALLEL_ATOMIC``); the Triton tile, warp
+    key raises ValueError.  Of the configuration, ``max_headdim``, ``exact_scale`` and the
+    ``SEQUENCE_PARALLEL`` and ``ATOMIC_DQ`` flags of the backward configurations are honoured (the
+    latter selects the atomic-add backward, ``GFX950_KERNEL_CONFIG_SEQUENCE_PARALLEL_ATOMIC``); the Triton tile, warp
     and stage counts are accepted and ignored (the reference hands them to its kernels, flash_attention_2.py:137-141;
     here the tile shapes are compiled in, one table row per padded head dimension).
 

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define FA2_ABI_VERSION 4
+#define FA2_ABI_VERSION 5
 
 /* Largest head dimension the kernels accept (the table's `max_headdim`). */
 #define FA2_MAX_HEADDIM 256
@@ -88,6 +88,13 @@ typedef struct fa2_config_info {
   int head_group;     /* (batch, head) pairs dispatched together; head_group / 8 share one XCD's L2 */
   int dq_atomic;      /* 1: sequence-parallel row - one backward kernel, dQ accumulated with fp32 global atomics
                          in a workspace (never picked by FA2_CONFIG_AUTO; selected by id) */
+  int fwd_exp_folded; /* 1: forward-only row.  The LDS-direct forward multiplies its Q fragments by
+                         softmax_scale * log2(e) and rounds them to the input type once, so that the score
+                         MFMAs deliver the base-2 exponents themselves (one vector instruction less per
+                         score; the reference scales the fp32 scores, _triton_kernels_v2.py:137-152).  O and
+                         lse are those of inputs whose Q is perturbed by at most half a unit in the last
+                         place.  Never picked by FA2_CONFIG_AUTO and refused by the backward entry points,
+                         which recompute the probabilities from Q itself; see fa2_pick_config_forward_only */
 } fa2_config_info;
 
 /* One (batch, nheads, seqlen, headdim) tensor: device pointer and strides in elements. */
@@ -144,9 +151,22 @@ int fa2_config_get(int config_id, fa2_config_info *out);
 
 /*
  * Table lookup: replaces _select_optimal_gpu_architecture (flash_attention_2.py:617-642).
- * Returns the row id (>= 0) chosen for the problem, or a negative fa2_status on error.
+ * Returns the row id (>= 0) that FA2_CONFIG_AUTO stands for, or a negative fa2_status on error.
+ * The row depends on the head dimension (the padded dimension the kernels are instantiated for).
+ * dtype, seqlen_q, seqlen_k and deterministic are validated and do not change the row: every row
+ * runs 128-row workgroups over 64-row streamed tiles in both types, and both backward modes run
+ * the same atomic-free kernels.
  */
 int fa2_pick_config(int dtype, int headdim, int seqlen_q, int seqlen_k, int deterministic);
+
+/*
+ * The row for a forward whose log-sum-exp no backward will read (inference, evaluation under
+ * no_grad): for bf16 up to 128 columns the row with fwd_exp_folded = 1, whose extra rounding of Q
+ * is of the size of the rounding bf16 inputs already carry; otherwise the row fa2_pick_config
+ * returns.  No counterpart in the reference, whose forward is the same in both situations
+ * (flash_attention_2.py:283-339).
+ */
+int fa2_pick_config_forward_only(int dtype, int headdim, int seqlen_q, int seqlen_k);
 
 /*
  * Forward: O = softmax(scale * Q K^T + causal mask) V and the row log-sum-exp.

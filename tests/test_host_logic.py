@@ -47,22 +47,38 @@ def test_abi_version_and_table(capi):
     lib = capi.load()
     assert lib.fa2_abi_version() == capi.ABI_VERSION
     rows = capi.config_table()
-    auto = [r for r in rows if not r["dq_atomic"]]  # the rows the table picks from by itself
-    assert [r["headdim_padded"] for r in auto] == sorted(r["headdim_padded"] for r in auto)
-    assert auto[-1]["headdim_padded"] == capi.FA2_MAX_HEADDIM
+    assert [r["id"] for r in rows] == list(range(len(rows)))
+    # The rows FA2_CONFIG_AUTO picks from (plain), and the forward-only rows whose forward folds the
+    # softmax scale into Q (what fa2_pick_config_forward_only returns for bf16 up to 128 columns).
+    plain = [r for r in rows if not r["dq_atomic"] and not r["fwd_exp_folded"]]
+    folded = [r for r in rows if r["fwd_exp_folded"]]
+    assert [r["headdim_padded"] for r in plain] == [32, 64, 96, 128, 192, 256]
+    assert [r["headdim_padded"] for r in folded] == [32, 64, 96, 128]
+    assert plain[-1]["headdim_padded"] == capi.FA2_MAX_HEADDIM
     for r in rows:
         assert r["fwd_block_q"] == 32 * r["fwd_waves"]
         assert r["bwd_block_kv"] == 32 * r["bwd_waves"]
         assert r["dq_block_q"] == 32 * r["dq_waves"]
+    by_dim = {r["headdim_padded"]: r for r in plain}
+    for r in folded:  # a folded row differs from the plain row of its head dimension in that flag only
+        twin = dict(by_dim[r["headdim_padded"]], id=r["id"], fwd_exp_folded=1)
+        assert r == twin and not r["dq_atomic"]
     for d, want in ((1, 32), (32, 32), (33, 64), (48, 64), (64, 64), (96, 96), (100, 128), (128, 128),
                     (129, 192), (192, 192), (193, 256), (256, 256)):
-        idx = lib.fa2_pick_config(capi.FA2_DTYPE_BF16, d, 512, 512, 0)
-        assert idx >= 0 and rows[idx]["headdim_padded"] == want
+        for dtype, seqlen in ((capi.FA2_DTYPE_F16, 512), (capi.FA2_DTYPE_BF16, 512), (capi.FA2_DTYPE_BF16, 16384)):
+            idx = lib.fa2_pick_config(dtype, d, seqlen, seqlen, 0)
+            assert idx >= 0 and rows[idx]["headdim_padded"] == want
+            assert not rows[idx]["dq_atomic"] and not rows[idx]["fwd_exp_folded"]
+            assert lib.fa2_pick_config(dtype, d, seqlen, seqlen, 1) == idx  # both backward modes share the row
+            only = lib.fa2_pick_config_forward_only(dtype, d, seqlen, seqlen)
+            assert only >= 0 and rows[only]["headdim_padded"] == want and not rows[only]["dq_atomic"]
+            assert rows[only]["fwd_exp_folded"] == int(dtype == capi.FA2_DTYPE_BF16 and want <= 128)
+    assert lib.fa2_pick_config_forward_only(capi.FA2_DTYPE_BF16, 257, 512, 512) == -4  # FA2_ERR_HEADDIM
     # LDS-direct kernels: all three up to 128 columns, forward and dQ only at 192 and 256.
-    assert [r["lds_direct"] for r in auto] == [1, 1, 1, 1, 2, 2]
+    assert [r["lds_direct"] for r in plain] == [1, 1, 1, 1, 2, 2]
     # (batch, head) pairs dispatched together: a multiple of 8 (one XCD per head), fewer at 128 columns.
     assert all(r["head_group"] % 8 == 0 and r["head_group"] > 0 for r in rows)
-    assert {r["headdim_padded"]: r["head_group"] for r in auto}[128] < {r["headdim_padded"]: r["head_group"] for r in auto}[64]
+    assert by_dim[128]["head_group"] < by_dim[64]["head_group"]
     assert lib.fa2_pick_config(capi.FA2_DTYPE_BF16, 257, 512, 512, 0) == -4  # FA2_ERR_HEADDIM
     assert lib.fa2_pick_config(7, 64, 512, 512, 0) == -3  # FA2_ERR_BAD_DTYPE
     info = capi.ConfigInfo()
@@ -129,6 +145,13 @@ def test_backward_entry_points_reject_bad_arguments(capi):
                      0.125, capi.FA2_DTYPE_F16, 1, capi.FA2_CONFIG_AUTO, None)
     assert lib.fa2_status_string(rc).decode() == "FA2_ERR_NULL_POINTER"
     assert "dv" in lib.fa2_last_error_string().decode()
+    # A forward-only row (its forward rounds Q * scale) is refused by the backward.
+    only = lib.fa2_pick_config_forward_only(capi.FA2_DTYPE_BF16, 64, 8, 8)
+    assert capi.config_table()[only]["fwd_exp_folded"] == 1
+    rc = lib.fa2_bwd(16, 16, 16, 16, 16, 16, None, 16, 16, 16, 1, 1, 8, 8, 64, 128, *(st * 7),
+                     0.125, capi.FA2_DTYPE_BF16, 1, only, None)
+    assert lib.fa2_status_string(rc).decode() == "FA2_ERR_BAD_CONFIG"
+    assert "forward-only" in lib.fa2_last_error_string().decode()
 
 
 def test_missing_library_fails_loudly(capi, monkeypatch, tmp_path):
@@ -147,15 +170,17 @@ def test_public_names_match_reference(fa):
 
 def test_kernels_config_is_a_frozen_record_with_reference_fields(fa):
     fields = [f.name for f in dataclasses.fields(fa.KernelsConfigV2)]
+    # The reference's nine fields in its order (_configurators_v2.py:27-38), then the one optional
+    # field this package adds; a configuration written for the reference constructs unchanged.
     assert fields == ["block_rows_size", "block_cols_size", "min_block_headdim", "max_headdim",
                       "seqlen_cache_divisor", "min_warps", "max_warps", "num_stages",
-                      "backward_autotune_configs"]
+                      "backward_autotune_configs", "exact_scale"]
     cfg = fa.KernelsConfigV2(128, 64, 32, 128, 32, 4, 4, 2, [
         fa.BackwardConfig({"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": False},
                           num_warps=4, num_stages=2, pre_hook=fa.init_to_zero_v2("DQ"))])
     with pytest.raises(dataclasses.FrozenInstanceError):
         cfg.block_rows_size = 64
-    assert cfg.deterministic is True
+    assert cfg.deterministic is True and cfg.exact_scale is False
     par = dataclasses.replace(cfg, backward_autotune_configs=[
         fa.BackwardConfig({"BLOCK_Q_ROWS_SIZE": 64, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": True})])
     assert par.deterministic is False

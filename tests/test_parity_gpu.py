@@ -296,6 +296,12 @@ def test_baseline_configs_match_oracle(fa, workloads, name):
         scale_ref = (q.cuda().float() * dq).abs().sum((-1, -2))
         assert ((lhs - rhs).abs() <= 2e-2 * scale_ref + 1e-2).all(), "sum(q*dq) != sum(k*dk)"
         torch.testing.assert_close(dv.sum(-2), d_o.cuda().float().sum(-2), atol=0.02 * math.sqrt(w.seqlen), rtol=2e-2)
+    # The forward that nothing will differentiate (for bf16 a forward-only row of the table).
+    with torch.no_grad():
+        out = fa.flash_attention_v2(q.cuda(), k.cuda(), v.cuda(), w.softmax_scale, False)
+    _assert_close(f"{name} o, forward only (cpu oracle)", flat(out)[:cpu_heads], cpu_want[0])
+    if gpu_want is not None:
+        _assert_close(f"{name} o, forward only (fp32 oracle on gpu)", out, gpu_want[0])
 
 
 def test_constant_values_give_constant_output(fa, workloads):
@@ -430,6 +436,61 @@ def test_custom_max_headdim_after_default_on_the_python_class(fa, fa2_module):
     out.backward(d_o.cuda())
     for name, a, b in zip(("o", "dq", "dk", "dv"), results[0], (out.detach(), qg.grad, kg.grad, vg.grad)):
         assert torch.equal(a, b), f"{name}: flash_attention_v2_custom(max_headdim=128) differs"
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 640, 640, 128), (2, 2, 333, 200, 48), (1, 4, 1024, 1024, 64), (1, 2, 77, 1, 64)],
+                         ids=lambda s: "B%dH%dNq%dNk%dD%d" % s)
+def test_forward_only_rows(fa, fa2_module, capi, shape):
+    """A forward that nothing will differentiate takes, for bf16 inputs, a table row whose kernel
+    folds softmax_scale * log2(e) into Q (rounded to bf16 once) instead of scaling the fp32 scores
+    as the reference does (_triton_kernels_v2.py:137-152).  Its O and lse must meet the parity
+    tolerance; a forward that a backward may follow, fp16 inputs, ``exact_scale`` configurations
+    and the plain row through the C ABI must all give the reference arithmetic's bits."""
+    b, h, nq, nk, d = shape
+    cc = torch.cuda.get_device_capability()
+    exact = {cc: fa.KernelsConfigV2(
+        block_rows_size=128, block_cols_size=64, min_block_headdim=32, max_headdim=256,
+        seqlen_cache_divisor=32, min_warps=4, max_warps=4, num_stages=2,
+        backward_autotune_configs=fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC.backward_autotune_configs,
+        exact_scale=True)}
+    lib = capi.load()
+    rows = capi.config_table()
+    for dtype, code in ((torch.bfloat16, capi.FA2_DTYPE_BF16), (torch.float16, capi.FA2_DTYPE_F16)):
+        q, k, v, d_o = _seeded((b, h, nq, d), (b, h, nk, d), dtype)
+        want = oracle.naive_causal_attention(q, k, v, None, torch.float32)
+        training = _run(fa, q, k, v, d_o, None, True)[0]
+        qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+        with torch.no_grad():
+            plain_inputs = fa.flash_attention_v2(qc, kc, vc)
+            no_grad = fa.flash_attention_v2(qc.requires_grad_(True), kc, vc)
+            exact_cfg = fa.flash_attention_v2_custom(qc, kc, vc, None, exact)
+        _assert_close(f"o, forward-only ({dtype})", no_grad, want)
+        assert torch.equal(no_grad, plain_inputs), "no_grad and inputs without requires_grad take the same row"
+        assert torch.equal(exact_cfg, training), "exact_scale must give the bits of the forward a backward follows"
+        only = rows[lib.fa2_pick_config_forward_only(code, d, nq, nk)]
+        auto = rows[lib.fa2_pick_config(code, d, nq, nk, 0)]
+        assert auto["fwd_exp_folded"] == 0 and only["headdim_padded"] == auto["headdim_padded"]
+        if dtype == torch.float16:
+            assert only["id"] == auto["id"] and torch.equal(no_grad, training)
+        else:
+            assert only["fwd_exp_folded"] == 1
+        # The same two rows by id through the C ABI, lse included.
+        n_r = math.ceil(nq / 128) * 128
+        s3 = fa2_module._strides3
+        st = torch.cuda.current_stream().cuda_stream
+        outs = {}
+        for row in (auto, only):
+            o = torch.empty_like(qc)
+            lse = torch.empty((b, h, n_r), dtype=torch.float32, device="cuda")
+            capi.check(lib.fa2_fwd(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(), lse.data_ptr(), b, h, nq,
+                                   nk, d, n_r, *s3(qc), *s3(kc), *s3(vc), *s3(o), 1.0 / math.sqrt(d), code, row["id"],
+                                   st), "fa2_fwd")
+            torch.cuda.synchronize()
+            outs[row["id"]] = (o, lse)
+        assert torch.equal(outs[auto["id"]][0], training) and torch.equal(outs[only["id"]][0], no_grad)
+        want_lse = oracle.naive_lse(q, k, None)
+        for row in (auto, only):
+            torch.testing.assert_close(outs[row["id"]][1][..., :nq].cpu(), want_lse, atol=2e-2, rtol=1e-2)
 
 
 def test_flash_attention_data_parallel(fa):
