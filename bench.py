@@ -193,10 +193,13 @@ def _kernel_legs(capi, w, q, k, v, d_o, iters: int):
     s3 = fa2._strides3
     stream = torch.cuda.current_stream().cuda_stream
 
-    def fwd():
+    def fwd(row=capi.FA2_CONFIG_AUTO):
         capi.check(lib.fa2_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
                                b, h, n, n, d, n_r, *s3(q), *s3(k), *s3(v), *s3(o),
-                               scale, dtype, capi.FA2_CONFIG_AUTO, stream), "fa2_fwd")
+                               scale, dtype, row, stream), "fa2_fwd")
+
+    # The row a forward takes that nothing will differentiate (what `fwd_ms` of the JSON line times).
+    forward_only_row = lib.fa2_pick_config_forward_only(dtype, d, n, n)
 
     def pre():
         capi.check(lib.fa2_bwd_preprocess(o.data_ptr(), d_o.data_ptr(), delta.data_ptr(), b, h, n, d, n_r,
@@ -207,6 +210,8 @@ def _kernel_legs(capi, w, q, k, v, d_o, iters: int):
     pre()
     torch.cuda.synchronize()
     results["fwd"] = _event_time_ms(fwd, iters)
+    results["fwd_forward_only"] = _event_time_ms(lambda: fwd(forward_only_row), iters)
+    fwd()  # leave the log-sum-exp of the forward a backward follows for the backward legs
     results["bwd_preprocess"] = _event_time_ms(pre, iters)
     ws_bytes = lib.fa2_bwd_workspace_bytes(b, h, n, n, d, 0, capi.FA2_CONFIG_AUTO)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=q.device)
@@ -463,12 +468,16 @@ def main() -> int:
     row_id = capi.load().fa2_pick_config(fa2._COMPUTE_DTYPES[w.dtype], w.headdim, w.seqlen, w.seqlen, int(det))
     row = capi.config_table()[row_id]
     kind = "direct_kernel" if row["lds_direct"] and row["headdim_padded"] == w.headdim else "kernel"
+    only_row = capi.config_table()[capi.load().fa2_pick_config_forward_only(fa2._COMPUTE_DTYPES[w.dtype], w.headdim,
+                                                                           w.seqlen, w.seqlen)]
     kernels = {
-        "fwd": (f"fwd_{kind} (fa2_fwd)", 1.0 * w.fwd_flops),
+        "fwd": (f"fwd_{kind} (fa2_fwd, table row {row['id']}: the forward a backward follows)", 1.0 * w.fwd_flops),
+        "fwd_forward_only": (f"fwd_{kind} (fa2_fwd, table row {only_row['id']}: the forward nothing differentiates, "
+                             "timed as fwd_ms)", 1.0 * w.fwd_flops),
         "bwd_dkdv": (f"bwd_dkdv_{kind} (fa2_bwd, dK/dV half)", 2.0 * w.fwd_flops),
         "bwd_dq": (f"bwd_dq_{kind} (fa2_bwd, dQ half)", 1.5 * w.fwd_flops),
     }
-    dominant = max(kernels, key=lambda name: leg_ms[name])
+    dominant = max((name for name in kernels if name != "fwd_forward_only"), key=lambda name: leg_ms[name])
     traffic, traffic_source = _measured_traffic(w.name)
 
     def mfma_roofline(name):
@@ -524,7 +533,8 @@ def main() -> int:
                    "sclk_mhz_during_fwd": fwd_clock.summary()},
         "settle_ms": args.settle_ms,
         "roofline": roofline,
-        "roofline_fwd": mfma_roofline("fwd"),
+        "roofline_fwd": mfma_roofline("fwd_forward_only"),
+        "roofline_fwd_in_step": mfma_roofline("fwd"),
         "roofline_bwd_dkdv": mfma_roofline("bwd_dkdv"),
         "roofline_bwd_dq": mfma_roofline("bwd_dq"),
         "bwd_tflops_algorithmic": bwd_tflops,
@@ -532,6 +542,7 @@ def main() -> int:
         "roofline_bwd_preprocess": pre_roofline,
         "kernel_ms": leg_ms,
         "table_row": row,
+        "table_row_forward_only": only_row,
     }
     if args.traffic_calibration:
         src = torch.ones(CALIBRATION_BYTES // 4, device=dev, dtype=torch.float32)

@@ -36,7 +36,7 @@ def build_torch_extension() -> pathlib.Path:
 def build(force: bool = True) -> pathlib.Path:
     """Compile the HIP kernels, the C ABI and the C++ autograd node.  ``force`` rebuilds even if
     the libraries exist."""
-    cmd = ["make", "-j4", "-C", str(CSRC)]
+    cmd = ["make", "-j5", "-C", str(CSRC)]
     if force:
         cmd.append("-B")
     subprocess.run(cmd, check=True)

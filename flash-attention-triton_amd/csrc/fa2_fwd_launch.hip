@@ -18,7 +18,10 @@ void launch_generic(int dp, const FwdParams &p, dim3 grid, dim3 block, hipStream
 }
 
 // PRE (exponents straight from the score MFMAs) is instantiated up to 128 columns: the sixteen registers
-// of the chain's start value are more than the 256-column kernel has left.
+// of the chain's start value are more than the 256-column kernel has left.  The 192- and 256-column
+// kernels live in a translation unit of their own (fa2_fwd_launch_wide.hip): compiled beside the
+// narrower instantiations the 256-column kernel, which uses all 512 registers, came out with 40-60
+// spilled registers and reloads inside its tile loop; alone it spills two, outside the loop.
 template <typename T, bool PAD, bool PRE>
 void launch_direct(int dp, const FwdParams &p, dim3 grid, dim3 block, hipStream_t s) {
   switch (dp) {
@@ -26,8 +29,7 @@ void launch_direct(int dp, const FwdParams &p, dim3 grid, dim3 block, hipStream_
     case 64: hipLaunchKernelGGL((fwd_direct_kernel<T, 64, kFwdBlockKV, PAD, PRE>), grid, block, 0, s, p); break;
     case 96: hipLaunchKernelGGL((fwd_direct_kernel<T, 96, kFwdBlockKV, PAD, PRE>), grid, block, 0, s, p); break;
     case 128: hipLaunchKernelGGL((fwd_direct_kernel<T, 128, kFwdBlockKV, PAD, PRE>), grid, block, 0, s, p); break;
-    case 192: hipLaunchKernelGGL((fwd_direct_kernel<T, 192, kFwdBlockKV, PAD, false>), grid, block, 0, s, p); break;
-    default: hipLaunchKernelGGL((fwd_direct_kernel<T, 256, kFwdBlockKV, PAD, false>), grid, block, 0, s, p); break;
+    default: launch_fwd_direct_wide(std::is_same<T, __bf16>::value, dp, PAD, p, grid, block, s); break;
   }
 }
 

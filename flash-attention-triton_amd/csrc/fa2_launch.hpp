@@ -57,6 +57,8 @@ inline int equal_head_groups(int group, int64_t heads) {
 // folded: the LDS-direct forward takes its exponents straight from the score MFMAs (Q fragments
 // multiplied by scale * log2(e) and rounded once); the generic forward ignores it.
 void launch_fwd(bool bf16, int dp, bool folded, const FwdParams &p, dim3 grid, hipStream_t s);
+// The 192- and 256-column LDS-direct forward kernels (dp is 192 or 256), instantiated apart from the others.
+void launch_fwd_direct_wide(bool bf16, int dp, bool pad, const FwdParams &p, dim3 grid, dim3 block, hipStream_t s);
 void launch_preprocess(bool bf16, const PreParams &p, dim3 grid, hipStream_t s);
 // fuse_delta: the fast dQ kernel also forms delta from O and dO (dq_direct_ok must hold).
 void launch_dq(bool bf16, int dp, const BwdParams &p, dim3 grid, bool fuse_delta, hipStream_t s);

@@ -17,9 +17,9 @@ TOOLS = [LLVM / "llvm-objcopy", LLVM / "clang-offload-bundler", LLVM / "llvm-rea
 LDS_PER_CU = 160 * 1024
 REGS_PER_LANE = 512  # VGPRs + accumulation registers per SIMD lane, shared by the waves on the SIMD
 
-# The one LDS-direct kernel that spills today: the forward at 256 columns without padding (its padded
-# twin fits).  Listed so that the number cannot grow unnoticed; the aim is zero.
-KNOWN_SPILLS = {("fwd_direct_kernel", 256, False): 64}
+# No LDS-direct kernel may spill.  (The forward at 256 columns is instantiated in its padded form only:
+# with the column count a compile-time 256 the compiler spilled about forty registers.)
+KNOWN_SPILLS: dict = {}
 
 
 def _kernel_records(library: pathlib.Path, tmp: pathlib.Path) -> list[dict]:
@@ -105,7 +105,7 @@ def test_registers_and_lds_leave_room_for_the_tables_workgroups(records):
     import importlib
 
     capi = importlib.import_module("flash-attention-triton_amd._capi")
-    rows = {r["headdim_padded"]: r for r in capi.config_table() if not r["dq_atomic"]}
+    rows = {r["headdim_padded"]: r for r in capi.config_table() if not r["dq_atomic"] and not r["fwd_exp_folded"]}
     column = {"fwd_direct_kernel": "fwd_wg_per_cu", "bwd_dq_direct_kernel": "dq_wg_per_cu",
               "bwd_dkdv_direct_kernel": "dkdv_wg_per_cu"}
     checked = 0
