@@ -45,13 +45,18 @@ METRIC = "causal attn TFLOP/s fwd & fwd+bwd (bf16, D=128) and % of MFMA peak, 1 
 
 
 def kernel_sources_hash() -> str:
-    """sha256 over the kernel sources (names and contents), the stamp the traffic summary carries."""
+    """sha256 over the kernel sources with comments and white space taken out (names and code): the
+    stamp the traffic summary carries.  A change of comments or layout leaves it alone; any change of
+    code, which may change the traffic, does not."""
     import hashlib
+    import re
 
+    strip = re.compile(r'//[^\n]*|/\*.*?\*/|("(?:\\.|[^"\\])*")', re.S)
     h = hashlib.sha256()
-    for path in sorted(KERNEL_SOURCES.glob("*.h*")):
+    for path in sorted(list(KERNEL_SOURCES.glob("*.h*")) + list(KERNEL_SOURCES.glob("Makefile"))):
+        text = strip.sub(lambda m: m.group(1) or " ", path.read_text())
         h.update(path.name.encode())
-        h.update(path.read_bytes())
+        h.update(" ".join(text.split()).encode())
     return h.hexdigest()[:16]
 
 

@@ -276,8 +276,11 @@ struct DkvDirectLayout {
   static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS + 4 * BQ;
   static constexpr int STAGES = 3;
   static constexpr int PATCH_ELEMS = kDkvWaves * 32 * (DP + 8);
-  static constexpr int TOTAL_ELEMS =
-      (STAGES * STAGE_ELEMS > PATCH_ELEMS) ? STAGES * STAGE_ELEMS : PATCH_ELEMS;
+  // Beyond the stages: room for the workgroup's 128 V rows on their way into registers (its K rows
+  // pass through the third stage before the third tile is requested).
+  static constexpr int V_ROWS_BASE = STAGES * STAGE_ELEMS;
+  static constexpr int TOTAL_ELEMS = V_ROWS_BASE + 2 * TILE_ELEMS;
+  static_assert(V_ROWS_BASE >= PATCH_ELEMS, "the output patch overlays the stages");
 };
 
 // PAD: the head dimension is a multiple of 8 below DP; the columns beyond it are zeros in LDS and in
@@ -335,7 +338,11 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 && !ATOMIC_DQ ? 2 : 1)) v
   const float *DELTA = p.delta + (int64_t)bh * p.seqlen_q_rounded;
 
   const int hdim = PAD ? p.headdim : DP;
-  const TileLoader<DP, BQ, kDkvWaves, PAD> qload(Q, p.q.stride_seq, hdim / 8), gload(DO, p.d_o.stride_seq, hdim / 8);
+  // (Bases and strides are restated as scalars: with the K and V loaders below in the same kernel the
+  // compiler otherwise forms the spread loads' addresses on the vector unit, 24 more vector
+  // instructions per tile.)
+  const TileLoader<DP, BQ, kDkvWaves, PAD> qload(uniform_ptr(Q), (int64_t)uniform64((uint64_t)p.q.stride_seq), hdim / 8),
+      gload(uniform_ptr(DO), (int64_t)uniform64((uint64_t)p.d_o.stride_seq), hdim / 8);
   const int seqlen_q = p.seqlen_q;
   const float scale_log2 = p.scale_log2;
 
@@ -348,7 +355,7 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 && !ATOMIC_DQ ? 2 : 1)) v
 
   const unsigned lds_base = lds_u32(smem);  // LDS byte address of smem
   if (PAD) {
-    zero_lds<NTHREADS>(smem, L::STAGES * L::STAGE_ELEMS);
+    zero_lds<NTHREADS>(smem, L::TOTAL_ELEMS);
     __syncthreads();
   }
   auto issue_tile = [&](int t) {
@@ -386,26 +393,26 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 && !ATOMIC_DQ ? 2 : 1)) v
       sl[BQ + tid] = -delta_reg;  // negated: it is the accumulator the dP MFMAs start from
     }
   };
-  // Prologue: every global load of the first three tiles and of this wave's K and V rows is
-  // issued before anything waits, so that the workgroup pays one memory latency, not one per
-  // tile.  (Tiles 1 and 2 cannot be requested later: the second block of tile 0 already fetches
-  // the first fragments of tile 1.)
-#pragma unroll
-  for (int t = 0; t < L::STAGES; t++)
-    if (t < n_tiles) issue_tile(t);
-
-  // B operands: lane (c, h) holds row kv0w + c of K and of V, columns 16 ks + 8 h + j.
-  s16x8 kf[KS], vf[KS];
+  // Prologue: the global loads of the first two tiles and of the workgroup's K and V rows are
+  // issued before anything waits, so that the workgroup pays one memory latency.  K and V travel
+  // like tiles: LDS-direct loads that cover whole rows, K into the third stage (whose tile is
+  // requested once every wave has taken its fragments out; it is first read near the end of tile 1),
+  // V behind the stages.  Loaded straight into registers, a wave's sixteen fragment loads touch 32
+  // rows each, and a workgroup, alone on its CU, spent 5 of its first 7 microseconds getting its
+  // loads accepted by the memory pipeline.  Rows beyond the keys are read from the last key row:
+  // finite values whose dK and dV rows are never stored.
+  constexpr unsigned K_LO = 2u * (unsigned)(2 * L::STAGE_ELEMS), K_HI = K_LO + 2u * (unsigned)L::TILE_ELEMS;
+  constexpr unsigned V_LO = 2u * (unsigned)L::V_ROWS_BASE, V_HI = V_LO + 2u * (unsigned)L::TILE_ELEMS;
   {
-    const int row = kv0w + c;
-    const bool ok = row < p.seqlen_k;
-    const short *kp = K + (int64_t)row * p.k.stride_seq;
-    const short *vp = V + (int64_t)row * p.v.stride_seq;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      kf[ks] = load_chunk(kp, 16 * ks + 8 * h, hdim, ok, true);
-      vf[ks] = load_chunk(vp, 16 * ks + 8 * h, hdim, ok, true);
-    }
+    const TileLoader<DP, BQ, kDkvWaves, PAD> kload(K + (int64_t)kv0 * p.k.stride_seq, p.k.stride_seq, hdim / 8),
+        vload(V + (int64_t)kv0 * p.v.stride_seq, p.v.stride_seq, hdim / 8);
+    const int k_rows = p.seqlen_k - kv0;  // key rows of this tile that exist (>= 1)
+    if (n_tiles > 0) issue_tile(0);
+    if (k_rows >= BQ) kload.issue(0, lds_base + K_LO); else kload.issue_clamped(0, k_rows, lds_base + K_LO);
+    if (k_rows >= 2 * BQ) kload.issue(BQ, lds_base + K_HI); else kload.issue_clamped(BQ, k_rows, lds_base + K_HI);
+    if (k_rows >= BQ) vload.issue(0, lds_base + V_LO); else vload.issue_clamped(0, k_rows, lds_base + V_LO);
+    if (k_rows >= 2 * BQ) vload.issue(BQ, lds_base + V_HI); else vload.issue_clamped(BQ, k_rows, lds_base + V_HI);
+    if (n_tiles > 1) issue_tile(1);
   }
   // B operands of the dQ GEMM: lane (c, h) holds column 32 (wave % DB) + c of K for the keys of key
   // group wave / DB, element j of k-step s being key 16 s + 8 (j / 4) + 4 h + j % 4 of the group (the
@@ -479,6 +486,22 @@ __global__ __launch_bounds__(64 * kDkvWaves, (DP <= 64 && !ATOMIC_DQ ? 2 : 1)) v
   }
   wait_vmem_all();
   __syncthreads();
+  // B operands: lane (c, h) holds row kv0w + c of K and of V, columns 16 ks + 8 h + j.
+  s16x8 kf[KS], vf[KS];
+  {
+    const int r = 32 * (wave & 1) + c;  // row inside the 64-row half the wave's keys lie in
+    const lds_cptr krows = lds0 + (int)(((wave >> 1) ? K_HI : K_LO) / 2);
+    const lds_cptr vrows = lds0 + (int)(((wave >> 1) ? V_HI : V_LO) / 2);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      kf[ks] = lds_read_128(krows + swz_off<LP>(r, 2 * ks + h));
+      vf[ks] = lds_read_128(vrows + swz_off<LP>(r, 2 * ks + h));
+    }
+  }
+  // Every wave has its K fragments: the third stage is free for its tile.
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (n_tiles > 2) issue_tile(2);
   // Two rings of A fragments, preloaded with the Q rows and the dO rows of block 0.
   s16x8 ring[KS], ringb[KS];
 #pragma unroll

@@ -311,6 +311,17 @@ __device__ __forceinline__ void load_lds_16(const short *uniform_base, unsigned 
       : "memory");
 }
 
+// A 64-bit value that is the same in every lane, moved to scalar registers.  For values whose
+// uniformity the compiler loses track of: address arithmetic on them then stays on the scalar unit.
+__device__ __forceinline__ uint64_t uniform64(uint64_t x) {
+  const uint64_t hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(x >> 32));
+  const uint64_t lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)x);
+  return (hi << 32) | lo;
+}
+__device__ __forceinline__ const short *uniform_ptr(const short *p) {
+  return (const short *)(uintptr_t)uniform64((uint64_t)(uintptr_t)p);
+}
+
 // s_waitcnt vmcnt(0) only (gfx9 encoding: expcnt and lgkmcnt fields left at their maxima).
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 // s_waitcnt vmcnt(N) only, 0 <= N < 64: wait until at most N vector-memory loads of this wave are

@@ -33,7 +33,8 @@ inline bool dq_direct_ok(int dp, const BwdParams &p) {
   return p.vec && direct_headdim_kv_stream(dp, p.headdim) && direct_stride_ok(p.k) && direct_stride_ok(p.v);
 }
 inline bool dkdv_direct_ok(int dp, const BwdParams &p) {
-  return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.q) && direct_stride_ok(p.d_o);
+  return p.vec && direct_headdim(dp, p.headdim) && direct_stride_ok(p.q) && direct_stride_ok(p.d_o) &&
+         direct_stride_ok(p.k) && direct_stride_ok(p.v);
 }
 // The sequence-parallel (atomic dQ) kernels: the fast dK/dV kernel's conditions, a head dimension
 // of exactly 32, 64 or 128 and 16-byte aligned dq rows.

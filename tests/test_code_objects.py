@@ -123,3 +123,32 @@ def test_registers_and_lds_leave_room_for_the_tables_workgroups(records):
         assert min(by_registers, by_lds) >= want, (r["name"], by_registers, by_lds, want)
         checked += 1
     assert checked >= 3 * 4 * 2
+
+
+# Two places in the kernels rest on facts about the compiler that no language rule guarantees: the
+# score chains of the dK/dV kernel are inline-assembly MFMAs whose results are made safe to read with
+# a hand-counted `s_nop 11` (the compiler's hazard recogniser does not see them), and the LDS-direct
+# loads write M0 from inline assembly without naming it as a clobber (the backend never keeps a value
+# in M0 across other code).  Both were validated, by reading the generated code and by the GPU parity
+# tests, with the compiler release named here; with another release they have to be looked at again
+# before this line is changed.
+VALIDATED_COMPILER = "roc-7.2.0"
+
+
+def test_hand_scheduled_code_was_validated_with_this_compiler():
+    hipcc = pathlib.Path("/opt/rocm/bin/hipcc")
+    if not hipcc.exists():
+        pytest.skip("no hipcc here")
+    out = subprocess.run([str(hipcc), "--version"], check=True, capture_output=True, text=True).stdout
+    assert VALIDATED_COMPILER in out, (
+        f"the kernels' hand-counted wait states (fa2_bwd_dkdv.hpp: VgprMfma, settle) and the unnamed M0 write "
+        f"(fa2_common.hpp: load_lds_16) were validated with {VALIDATED_COMPILER}; this compiler reports:\n{out}")
+
+
+def test_hand_counted_wait_states_are_in_the_code(records, tmp_path):
+    """The dK/dV kernel's inline-assembly MFMA chains must still be followed by their `s_nop 11`
+    before the first vector instruction reads them: one per chain and 32-row block in the source."""
+    src = (pathlib.Path(__file__).resolve().parent.parent / "flash-attention-triton_amd" / "csrc" /
+           "fa2_bwd_dkdv.hpp").read_text()
+    assert src.count('asm volatile("s_nop 11" : "+v"(d))') == 1
+    assert src.count("settle(s)") == 1 and src.count("settle(dp)") == 1
