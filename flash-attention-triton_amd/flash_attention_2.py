@@ -573,6 +573,35 @@ def flash_attention_v2(
     return _apply(q, k, v, softmax_scale, kernels_config)
 
 
+_TILE_WARNING_SHOWN = False
+
+
+def _warn_about_ignored_tile_fields(kernels_config: KernelsConfigV2) -> None:
+    """Say once when a custom configuration asks for tile shapes other than the compiled ones.
+
+    The reference hands these values to its kernels (flash_attention_2.py:137-141, 773-790); the
+    gfx950 kernels exist in one tile shape per table row, so other values cannot be honoured."""
+    global _TILE_WARNING_SHOWN
+    if _TILE_WARNING_SHOWN:
+        return
+    compiled = GFX950_KERNEL_CONFIG_DETERMINISTIC
+    asked = (kernels_config.block_rows_size, kernels_config.block_cols_size, kernels_config.min_warps)
+    have = (compiled.block_rows_size, compiled.block_cols_size, compiled.min_warps)
+    backward = [(c.kwargs.get("BLOCK_Q_ROWS_SIZE"), c.kwargs.get("BLOCK_KV_COLS_SIZE"))
+                for c in kernels_config.backward_autotune_configs if hasattr(c, "kwargs")]
+    have_bwd = (compiled.backward_autotune_configs[0].kwargs["BLOCK_Q_ROWS_SIZE"],
+                compiled.backward_autotune_configs[0].kwargs["BLOCK_KV_COLS_SIZE"])
+    if asked != have or any(b != have_bwd and b != (None, None) for b in backward):
+        import warnings
+
+        _TILE_WARNING_SHOWN = True
+        warnings.warn(
+            f"flash_attention_v2_custom: the gfx950 kernels are compiled for {have[0]}-row workgroups over "
+            f"{have[1]}-row streamed tiles with {have[2]} wavefronts (backward {have_bwd[0]} x {have_bwd[1]}); the "
+            f"configuration asks for {asked} (backward {backward}) and these fields are ignored.  max_headdim, "
+            "exact_scale, SEQUENCE_PARALLEL and ATOMIC_DQ are honoured.", stacklevel=3)
+
+
 def flash_attention_v2_custom(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -609,6 +638,7 @@ def flash_attention_v2_custom(
     _validate_runtime_compatibility(cc)
 
     kernels_config = kernels_configs[cc]
+    _warn_about_ignored_tile_fields(kernels_config)
     if kernels_config.max_headdim > _capi.FA2_MAX_HEADDIM:
         raise ValueError(
             f"max_headdim={kernels_config.max_headdim} exceeds what the compiled kernels "

@@ -211,6 +211,25 @@ def test_selector_and_validation(fa2_module, monkeypatch):
         fa2_module.flash_attention_v2_custom(q, q, q, None, {(8, 0): sel((9, 5), True)})
 
 
+def test_custom_tile_fields_are_reported_not_silently_dropped(fa, fa2_module, monkeypatch):
+    """The reference passes a custom configuration's tile and warp values to its kernels
+    (flash_attention_2.py:137-141); here they cannot change the compiled kernels, and the caller is
+    told so once.  The compiled shapes themselves raise no warning."""
+    import warnings
+
+    monkeypatch.setattr(fa2_module, "_TILE_WARNING_SHOWN", False)
+    ampere = fa.KernelsConfigV2(256, 256, 32, 256, 32, 8, 8, 1, [
+        fa.BackwardConfig({"BLOCK_Q_ROWS_SIZE": 128, "BLOCK_KV_COLS_SIZE": 128, "SEQUENCE_PARALLEL": False})])
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        fa2_module._warn_about_ignored_tile_fields(fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC)
+        fa2_module._warn_about_ignored_tile_fields(fa2_module.GFX950_KERNEL_CONFIG_SEQUENCE_PARALLEL_ATOMIC)
+        assert not seen
+        fa2_module._warn_about_ignored_tile_fields(ampere)
+        fa2_module._warn_about_ignored_tile_fields(ampere)
+    assert len(seen) == 1 and "ignored" in str(seen[0].message) and "exact_scale" in str(seen[0].message)
+
+
 def test_launcher_assertions_mirror_reference(fa2_module):
     """Same AssertionErrors as flash_attention_2.py:85-90, raised before any FFI call."""
     cfg = fa2_module.GFX950_KERNEL_CONFIG_DETERMINISTIC
