@@ -530,6 +530,10 @@ def main() -> int:
         "fwd_tflops": fwd_tflops,
         "fwd_ms": fwd_ms,
         "fwd_frac_of_peak": fwd_tflops / peak,
+        # fwd_ms times the public function under torch.no_grad(): for bf16 that is the forward-only
+        # table row.  The forward inside the timed step (a backward follows) is the plain row:
+        "fwd_in_step_kernel_ms": leg_ms["fwd"],
+        "fwd_in_step_frac_of_peak": w.fwd_flops / (leg_ms["fwd"] * 1e-3) / 1e12 / peak,
         "peak_tflops": peak,
         "device": {"name": props.name, "arch": getattr(props, "gcnArchName", ""),
                    "compute_units": props.multi_processor_count,
