@@ -369,10 +369,15 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=50, help="untimed steps right before the timed ones")
     ap.add_argument("--settle-ms", type=float, default=400.0,
-                    help="before the warm-up steps, run untimed steps for this long: an idle GPU sits at "
-                         "~100 MHz and its clocks and power controller need some hundreds of milliseconds of "
-                         "load to reach the steady state a training job runs in (the first 20 steps after 5 "
-                         "warm-up steps measure 5-6 %% slower than steady state)")
+                    help="before the warm-up steps, run untimed steps for at least this long and then until "
+                         "their rate has stopped changing (see --settle-max-ms): an idle GPU sits at ~100 MHz, "
+                         "its clocks need some hundreds of milliseconds of load, and under its power limit the "
+                         "chip keeps getting faster for several seconds as it warms up (on a box that had been "
+                         "idle the same 20 steps measured 6 %% slower after 0.4 s of load than after 8 s).  "
+                         "0 switches the phase off")
+    ap.add_argument("--settle-max-ms", type=float, default=20000.0,
+                    help="upper bound of the settle phase; it ends earlier once the rate of half-second windows "
+                         "of calls has stopped moving (last three within 0.4 %%, less than 0.3 %% over two seconds)")
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--deterministic", action="store_true", help="time the deterministic backward in the step")
     ap.add_argument("--cpu-heads", type=int, default=64, help="(batch, head) slices in the CPU baseline sample")
@@ -414,13 +419,31 @@ def main() -> int:
             return pkg.flash_attention_v2(q, k, v, scale, det)
 
     def settle(fn):
-        t_end = time.perf_counter() + args.settle_ms * 1e-3
-        while time.perf_counter() < t_end:
-            for _ in range(10):
-                fn()
-            torch.cuda.synchronize()
+        """Untimed calls until the rate is steady (at least --settle-ms, at most --settle-max-ms).
+        Returns what was observed."""
+        if args.settle_ms <= 0:
+            return {"ms": 0.0, "windows": 0}
+        t_begin = time.perf_counter()
+        windows = []
+        while True:
+            t0, calls = time.perf_counter(), 0
+            while time.perf_counter() - t0 < 0.5:
+                for _ in range(10):
+                    fn()
+                torch.cuda.synchronize()
+                calls += 10
+            windows.append((time.perf_counter() - t0) * 1e3 / calls)
+            elapsed_ms = (time.perf_counter() - t_begin) * 1e3
+            # Steady: the last three windows agree within 0.4 % and the rate has moved by less than
+            # 0.3 % over the last two seconds (the warm-up drift is slow: a tenth of a percent a second).
+            last = windows[-3:]
+            steady = (len(windows) >= 5 and max(last) / min(last) - 1.0 < 0.004
+                      and abs(windows[-1] / windows[-5] - 1.0) < 0.003)
+            if elapsed_ms >= args.settle_max_ms or (elapsed_ms >= args.settle_ms and steady):
+                return {"ms": elapsed_ms, "windows": len(windows), "first_window_ms_per_call": windows[0],
+                        "last_window_ms_per_call": windows[-1]}
 
-    settle(step)
+    settle_step = settle(step)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -445,7 +468,7 @@ def main() -> int:
         torch.cuda.synchronize()
         step_ms_one_thread = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    settle(fwd_only)
+    settle_fwd = settle(fwd_only)
     for _ in range(max(args.warmup, 1)):
         fwd_only()
     torch.cuda.synchronize()
@@ -540,7 +563,10 @@ def main() -> int:
                    "clock_mhz": _device_clock_mhz(props),
                    "sclk_mhz_during_steps": step_clock.summary(),
                    "sclk_mhz_during_fwd": fwd_clock.summary()},
-        "settle_ms": args.settle_ms,
+        # Untimed calls before each timed region (forward + backward steps, then forward only) and how
+        # their rate moved meanwhile; see --settle-ms.
+        "settle_ms": settle_step["ms"] + settle_fwd["ms"],
+        "settle": {"steps": settle_step, "fwd": settle_fwd},
         "roofline": roofline,
         "roofline_fwd": mfma_roofline("fwd_forward_only"),
         "roofline_fwd_in_step": mfma_roofline("fwd"),
