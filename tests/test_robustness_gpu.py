@@ -125,6 +125,10 @@ def test_randomised_shape_sweep(fa):
         got = _run(fa, q, k, v, d_o, scale, deterministic)
         for name, g, w in zip(("o", "dq", "dk", "dv"), got, want):
             _assert_close(f"{label}: {name}", g, w)
+        # The same forward with nothing to differentiate (bf16 up to 128 columns: a forward-only row).
+        with torch.no_grad():
+            out = fa.flash_attention_v2(q.cuda(), k.cuda(), v.cuda(), scale, deterministic)
+        _assert_close(f"{label}: o, forward only", out, want[0])
 
 
 # ---------------------------------------------------------------- lse at the long and the peaky sizes
