@@ -332,3 +332,28 @@ def test_workload_table_matches_baseline(workloads):
     q2, *_ = workloads.make_inputs(w["C1"], heads=3)
     assert q.dtype == torch.float16 and q.shape == (2, 4, 512, 64)
     torch.testing.assert_close(q2[:, 0], q.reshape(8, 512, 64)[:3], atol=0, rtol=0)
+
+
+def test_traffic_stamp_ignores_comments_and_follows_code(tmp_path, monkeypatch):
+    """bench.py drops the measured HBM traffic when the kernel sources have changed since the
+    counter run.  The stamp it compares must not move when comments or layout change (nobody should
+    have to re-stamp a summary by hand) and must move when code does."""
+    import importlib
+
+    bench = importlib.import_module("bench")
+    src = tmp_path / "csrc"
+    src.mkdir()
+    (src / "k.hpp").write_text('// a comment\nint f(int x) { return x + 1; }  /* tail */\nconst char *s = "// not a comment";\n')
+    (src / "Makefile").write_text("all:\n\ttrue\n")
+    monkeypatch.setattr(bench, "KERNEL_SOURCES", src)
+    base = bench.kernel_sources_hash()
+    (src / "k.hpp").write_text('// another comment, more of it\n\nint f(int x)\n{\n  return x + 1;\n}\nconst char *s = "// not a comment";\n')
+    assert bench.kernel_sources_hash() == base
+    (src / "k.hpp").write_text('int f(int x) { return x + 2; }\nconst char *s = "// not a comment";\n')
+    assert bench.kernel_sources_hash() != base
+    (src / "k.hpp").write_text('int f(int x) { return x + 1; }\nconst char *s = "// not a comment!";\n')
+    assert bench.kernel_sources_hash() != base
+    # The committed summary carries the stamp of the committed sources.
+    monkeypatch.undo()
+    rows, source = bench._measured_traffic("C3")
+    assert rows.get("fwd") and rows.get("bwd_dkdv") and rows.get("fwd_forward_only"), source
